@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Flash-decode benchmark: one decode step = split-KV GQA paged decode + LSE combine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 100] [--warmup 20] [--config 2]
+
+Prints ONE JSON line.  ``value`` is microseconds per decode step with all inputs resident in
+HBM; the step rotates over several independent KV pools so the 256 MB Infinity Cache cannot
+serve the working set.  ``roofline`` prices the split-KV kernel (the dominant one) against
+the 8 TB/s HBM peak with the algorithmic bytes of a step; ``cpu_baseline`` is the CPU oracle
+(the reference's PyTorch decode restated) timed on this host's cores on the same inputs.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, help="BASELINE.json configs, 1-based (2 = Llama-3-8B shape)")
+    ap.add_argument("--pools", type=int, default=4, help="independent KV pools the steps rotate over")
+    ap.add_argument("--variant", default="plain", choices=["plain", "persistent"])
+    ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
+    ap.add_argument("--waves", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
+    ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    fd = importlib.import_module("triton-distributed_amd")
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the flash-decode library has no CPU path", file=sys.stderr)
+        sys.exit(2)
+    fd.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    wl_cpu = fd.utils.make_config5_bf16_twin() if args.bf16_twin else fd.utils.make_config(args.config)
+    wl = wl_cpu.to(dev)
+    B, Hq, D = wl.q.shape
+    S = wl.kv_split
+    algo_bytes = wl_cpu.algorithmic_bytes()
+
+    # independent KV pools: pool 0 holds the seeded data (checked against the CPU baseline), the
+    # others hold other random bits of the same distribution
+    pools = [(wl.k_cache, wl.v_cache)]
+    for i in range(1, max(1, args.pools)):
+        if wl.k_cache.dtype in (torch.float16, torch.bfloat16, torch.float32):
+            k = torch.empty_like(wl.k_cache).normal_()
+            v = torch.empty_like(wl.v_cache).normal_()
+        else:  # fp8 bit patterns: shuffle pages of pool 0
+            perm = torch.randperm(wl.k_cache.shape[0], device=dev)
+            k = wl.k_cache[perm].contiguous()
+            v = wl.v_cache[perm].contiguous()
+        pools.append((k, v))
+
+    out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
+    lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
+    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev)
+    q_lens = [1] * B
+    kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=args.path, waves_per_block=args.waves)
+    if wl.k_scale is not None:
+        kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
+    if wl.extra_out is not None:
+        kw.update(extra_partials=(wl.extra_out, wl.extra_lse))
+    fn = fd.gqa_fwd_batch_decode_persistent if args.variant == "persistent" else fd.gqa_fwd_batch_decode
+    if args.variant == "persistent":
+        kw["seq_order"] = torch.empty(B, dtype=torch.int32, device=dev)
+
+    def step(i):
+        k, v = pools[i % len(pools)]
+        if args.variant == "persistent":   # the scheduler is part of the step
+            fd.schedule_sequences(wl.kv_lens, out=kw["seq_order"])
+        return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
+
+    # ---- whole-step timing
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = e0.elapsed_time(e1)
+    ms_per_step = max(gpu_ms, 0.0) / args.steps
+    us_per_step = ms_per_step * 1e3
+
+    # ---- dominant kernel alone (split-KV), HIP events on the launch stream
+    from ctypes import byref
+    lib = fd.load_library()
+    fk = importlib.import_module("triton-distributed_amd.kernels.flash_decode")
+    n_o = B * Hq * S * D
+    mid = workspace[:n_o].view(B, Hq, S, D)
+    lse_split = workspace[n_o:n_o + B * Hq * S].view(B, Hq, S)
+    p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
+                        wl.k_scale, wl.v_scale, args.path, args.waves)
+    hstream = torch.cuda.current_stream().cuda_stream
+    order_ptr = kw["seq_order"].data_ptr() if args.variant == "persistent" else None
+
+    def split_only(i):
+        k, v = pools[i % len(pools)]
+        fd._lib.check(lib.fd_split_kv(
+            hstream, wl.q.data_ptr(), k.data_ptr(), v.data_ptr(), mid.data_ptr(), lse_split.data_ptr(),
+            float(wl.scale), wl.block_table.data_ptr(), wl.kv_lens.data_ptr(), B,
+            wl.q.stride(0), wl.q.stride(1), k.stride(-3), k.stride(-2), v.stride(-3), v.stride(-2),
+            mid.stride(0), mid.stride(1), mid.stride(2), wl.block_table.stride(0), order_ptr, byref(p)))
+
+    for i in range(args.warmup):
+        split_only(i)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(args.steps):
+        split_only(i)
+    e1.record()
+    torch.cuda.synchronize()
+    split_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    achieved = algo_bytes / (split_us * 1e-6) / 1e9
+
+    # ---- result of pool 0 for the check against the CPU baseline
+    step(0)
+    torch.cuda.synchronize()
+    out_gpu, lse_gpu = out.float().cpu(), lse.cpu()
+
+    result = {
+        "metric": "us/decode step + achieved HBM GB/s (% of 8 TB/s), GQA paged decode, 1 GPU",
+        "value": round(us_per_step, 3),
+        "unit": "us/decode step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8-e4m3 KV / bf16 Q, fp32 accumulate" if wl.k_scale is not None else
+                 f"{str(wl.q.dtype).replace('torch.', '')} KV+Q, fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": wl.name, "batch": B, "q_heads": Hq, "kv_heads": wl.k_cache.shape[2], "head_dim": D,
+                   "page_size": wl.k_cache.shape[1], "kv_splits": S,
+                   "kv_len_total": int(wl_cpu.kv_lens.sum()), "kv_pools_rotated": len(pools),
+                   "variant": args.variant, "path": args.path},
+        "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),
+        "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
+        "algorithmic_bytes": algo_bytes,
+        "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel_us": round(split_us, 3)},
+    }
+
+    if not args.no_cpu_baseline:
+        import oracle  # the checker, timed as the CPU baseline only
+        n_seq = args.cpu_seqs or (B if algo_bytes < 6e8 else max(1, min(B, 4)))
+        rows = list(range(n_seq))
+        torch_threads = torch.get_num_threads()
+        lens = [int(x) for x in wl_cpu.kv_lens.tolist()]
+        P = wl_cpu.k_cache.shape[1]
+        used = torch.unique(torch.cat([wl_cpu.block_table[i, :-(-lens[i] // P)].long() for i in rows]))
+        remap = torch.zeros(wl_cpu.k_cache.shape[0], dtype=torch.long)
+        remap[used] = torch.arange(used.numel())
+        bt = torch.zeros_like(wl_cpu.block_table[rows])
+        for j, i in enumerate(rows):
+            npg = -(-lens[i] // P)
+            bt[j, :npg] = remap[wl_cpu.block_table[i, :npg].long()].to(torch.int32)
+        kc, vc = wl_cpu.k_cache[used], wl_cpu.v_cache[used]
+        if wl_cpu.k_scale is not None:
+            kc = oracle.dequant_fp8_cache(kc.view(torch.uint8), wl_cpu.k_scale)
+            vc = oracle.dequant_fp8_cache(vc.view(torch.uint8), wl_cpu.v_scale)
+        kc, vc, qc = kc.float(), vc.float(), wl_cpu.q[rows].float()
+        sub_lens = [lens[i] for i in rows]
+        times = []
+        ref = ref_lse = None
+        for it in range(4):  # 1 warm-up + 3 timed
+            t = time.perf_counter()
+            ref, ref_lse = oracle.ref_paged_attn_lse(qc, kc, vc, sub_lens, bt, wl_cpu.scale, soft_cap=wl_cpu.soft_cap)
+            if it:
+                times.append(time.perf_counter() - t)
+        frac_tokens = sum(sub_lens) / max(1, sum(lens))
+        cpu_us = statistics.median(times) * 1e6 / frac_tokens
+        if wl_cpu.extra_out is None:
+            err_o = (out_gpu[rows] - ref).abs().max().item()
+            fin = torch.isfinite(ref_lse)
+            err_l = ((lse_gpu[rows] - ref_lse)[fin].abs() / ref_lse[fin].abs().clamp_min(1.0)).max().item()
+            result["check_vs_cpu_baseline"] = {"max_abs_err_out": round(err_o, 6), "max_rel_err_lse": round(err_l, 8)}
+        result["cpu_baseline"] = {
+            "value": round(cpu_us, 1), "unit": "us/decode step", "cores": torch_threads, "kind": "port",
+            "sample": f"oracle.ref_paged_attn_lse (fp32 PyTorch restatement of the reference's ref_paged_attn) on "
+                      f"sequences 0..{n_seq - 1} of {B} of the same seeded workload, median of 3 runs, scaled by "
+                      f"1/{frac_tokens:.4f} (token share) to the whole step; host cpu_count={os.cpu_count()}",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,179 @@
+/*
+ * flash_decode.h -- C ABI of the MI355X (gfx950) flash-decode library.
+ *
+ * One shared library, libflash_decode_gfx950.so, exports exactly the symbols
+ * declared here.  All pointers are DEVICE pointers (tensor.data_ptr()), all
+ * strides are in ELEMENTS and 64-bit, `stream` is a hipStream_t passed as
+ * void* (NULL = the legacy default stream).  Every call only enqueues work on
+ * `stream`; nothing synchronises with the host and kv_lens is never read on the
+ * host.  Return value: 0 on success, a negative fd_status otherwise;
+ * fd_last_error() then describes the failure for the calling thread.  The
+ * library never aborts the process.
+ *
+ * The shape of this ABI follows what the reference generates for its
+ * ahead-of-time compiled Triton kernels: `CUresult <kernel>_ex(CUstream,
+ * <pointers, scalars, strides...>, struct algo_info)`
+ * (python/triton_dist/tools/compile_aot.py:330-333, 405-435), with the argument
+ * order of the Triton signatures in
+ * python/triton_dist/kernels/nvidia/flash_decode.py:70-94 (split) and :242-276
+ * (combine).  The reference's pybind lambda drops the return code
+ * (compile_aot.py:375-379); here it is returned to the caller.
+ */
+#ifndef FLASH_DECODE_H_
+#define FLASH_DECODE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FD_ABI_VERSION 1
+
+#if defined(__GNUC__)
+#define FD_API __attribute__((visibility("default")))
+#else
+#define FD_API
+#endif
+
+typedef enum fd_status {
+  FD_OK = 0,
+  FD_ERR_INVALID_ARG = -1,  /* NULL pointer, non-positive size, bad enum            */
+  FD_ERR_UNSUPPORTED = -2,  /* dtype / head_dim / group combination not compiled   */
+  FD_ERR_ALIGNMENT = -3,    /* pointer or stride not aligned for 128-bit accesses  */
+  FD_ERR_LAUNCH = -4,       /* the HIP runtime refused the launch                  */
+  FD_ERR_TOO_LARGE = -5     /* size beyond a documented maximum                    */
+} fd_status;
+
+typedef enum fd_dtype {
+  FD_F32 = 0,
+  FD_F16 = 1,
+  FD_BF16 = 2,
+  FD_FP8_E4M3 = 3           /* OCP e4m3fn bit patterns, KV cache only              */
+} fd_dtype;
+
+typedef enum fd_path {
+  FD_PATH_AUTO = 0,         /* MFMA when group >= 4, 16-bit/fp8 KV, head_dim 128   */
+  FD_PATH_VALU = 1,         /* force the VALU dot-product kernel                   */
+  FD_PATH_MFMA = 2          /* force MFMA; FD_ERR_UNSUPPORTED if not applicable    */
+} fd_path;
+
+typedef enum fd_combine_mode {
+  FD_COMBINE_SPLIT = 0,     /* validity by split range, flash_decode.py:339-343    */
+  FD_COMBINE_SPLIT_LSE = 1, /* same + merged LSE at column Dv of the output row,
+                               flash_decode.py:446-449                             */
+  FD_COMBINE_RANK = 2       /* validity by seqlens[s*batch+b] > 0,
+                               flash_decode.py:513-515                             */
+} fd_combine_mode;
+
+/*
+ * Compile-time constants of the reference's Triton kernels (kv_group_num,
+ * q_head_num, NUM_KV_SPLITS, PAGE_SIZE, soft_cap, K_DIM, V_DIM --
+ * flash_decode.py:153-164; the `algo_info` struct of the AOT path,
+ * flash_decode.py:103-109) plus what a typed C ABI needs to know about the
+ * buffers.  Zero-initialise, then fill.
+ */
+typedef struct fd_params {
+  int32_t q_heads;          /* Hq                                                  */
+  int32_t kv_heads;         /* Hkv; Hq % Hkv == 0                                  */
+  int32_t head_dim;         /* Dk == Dv; 64, 128 or 256                            */
+  int32_t page_size;        /* tokens per page (any value >= 1)                    */
+  int32_t num_splits;       /* NUM_KV_SPLITS                                       */
+  int32_t num_pages;        /* pages in the pool: table entries are clamped to
+                               [0, num_pages) before use                           */
+  int32_t max_pages_per_seq;/* block_table.shape[1]; kv_len is clamped to
+                               max_pages_per_seq * page_size                       */
+  int32_t q_dtype;          /* fd_dtype of q                                       */
+  int32_t kv_dtype;         /* fd_dtype of k_cache / v_cache                       */
+  int32_t mid_dtype;        /* fd_dtype of the split partials (out_split / mid_o)  */
+  int32_t out_dtype;        /* fd_dtype of the combined output                     */
+  float soft_cap;           /* <= 0: off                                           */
+  const float* k_scale;     /* [Hkv] fp32 dequant scales, FD_FP8_E4M3 only         */
+  const float* v_scale;     /* [Hkv]                                               */
+  int32_t path;             /* fd_path                                             */
+  int32_t waves_per_block;  /* 0 = choose; else 1, 2, 4 or 8 wave64 per workgroup  */
+} fd_params;
+
+/*
+ * Kernel (1): split-KV GQA paged decode.
+ * Replaces kernel_gqa_fwd_batch_decode_split_kv
+ * (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) and its launch
+ * (flash_decode.py:788-824 grid/arguments).
+ *
+ *  q           [batch, Hq, D]            stride_q_bs, stride_q_h, last dim contiguous
+ *  k_cache     [num_pages, P, Hkv, D]    stride_k_tok = stride(-3), stride_k_h = stride(-2);
+ *                                        the pool is indexed by flat token row page*P + n%P
+ *  v_cache     same with stride_v_*
+ *  out_split   [batch, Hq, S, *]         normalised partial outputs, mid_dtype, strides
+ *                                        stride_o_bs / stride_o_h / stride_o_split
+ *  lse_split   NULL: partial LSE (natural log) is stored at column D of the out_split row
+ *              (the reference layout [B,Hq,S,D+1]); else fp32 [batch, Hq, S] contiguous
+ *  block_table [batch, max_pages] int32, row stride stride_table_bs; only the first
+ *              ceil(kv_len/P) entries of a row are read
+ *  seq_order   NULL, or [batch] int32 from fd_schedule: workgroups are issued in this
+ *              sequence order (longest first)
+ *
+ * Split s of sequence b covers tokens [per*s, min(per*s+per, kv_len)), per =
+ * ceil(kv_len/S).  An empty split stores out = 0, lse = -inf.
+ */
+FD_API int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                void* out_split, float* lse_split, float sm_scale,
+                const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
+                int64_t stride_q_bs, int64_t stride_q_h,
+                int64_t stride_k_tok, int64_t stride_k_h,
+                int64_t stride_v_tok, int64_t stride_v_h,
+                int64_t stride_o_bs, int64_t stride_o_h, int64_t stride_o_split,
+                int64_t stride_table_bs,
+                const int32_t* seq_order, const fd_params* params);
+
+/*
+ * Kernel (2): LSE-weighted combine.  One entry point covers the reference's
+ * three combine kernels:
+ *   FD_COMBINE_SPLIT      kernel_gqa_fwd_batch_decode_combine_kv            flash_decode.py:308-360
+ *   FD_COMBINE_SPLIT_LSE  kernel_intra_rank_gqa_fwd_batch_decode_combine_kv flash_decode.py:393-449
+ *   FD_COMBINE_RANK       kernel_inter_rank_gqa_fwd_batch_decode_combine_kv flash_decode.py:482-532
+ *                         as launched by layers/nvidia/sp_flash_decode_layer.py:173-183
+ *
+ *  mid_o     partials, params->mid_dtype, element strides stride_mid_ob (batch),
+ *            stride_mid_oh (head), stride_mid_os (split or rank); `num_partials` of them
+ *            (params->num_splits is ignored here)
+ *  mid_lse   NULL: LSE of a partial is at column D of its mid_o row; else fp32 with
+ *            contiguous layout [batch, Hq, num_partials]
+ *  out       [batch, Hq, D(+1)] params->out_dtype, strides stride_obs / stride_oh
+ *  lse_out   NULL or fp32 [batch, Hq]: merged natural-log LSE (always fp32)
+ *  seqlens   kv_lens [batch] (split modes) or global_kv_lens [num_partials, batch] (rank mode)
+ *  extra_out / extra_lse / num_extra
+ *            further always-valid partials merged in the same pass:
+ *            extra_out [num_extra, batch, Hq, D] contiguous in params->out_dtype,
+ *            extra_lse [num_extra, batch, Hq] fp32.  They stand in, on one GPU, for the
+ *            partials the reference's allgather delivers from other ranks
+ *            (sp_flash_decode_layer.py:136-145).
+ *
+ * A row with no valid partial yields out = 0, lse = -inf (the reference yields NaN).
+ */
+FD_API int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
+               const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials,
+               int64_t stride_mid_ob, int64_t stride_mid_oh, int64_t stride_mid_os,
+               int64_t stride_obs, int64_t stride_oh, int32_t mode,
+               const void* extra_out, const float* extra_lse, int32_t num_extra,
+               const fd_params* params);
+
+/*
+ * Kernel (3): work scheduler.  Writes seq_order[batch]: sequence indices sorted by
+ * kv_len descending (ties by index), computed on the device from kv_lens, so that
+ * fd_split_kv issues the longest sequences' workgroups first and the hardware
+ * dispatcher back-fills CUs with the short ones.  The reference's only scheduler is
+ * the static round-robin of its persistent kernel (flash_decode.py:632-640).
+ */
+FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* seq_order);
+
+/* Message for the last non-zero status returned on this thread ("" if none). */
+FD_API const char* fd_last_error(void);
+
+/* FD_ABI_VERSION the library was built with. */
+FD_API int fd_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_DECODE_H_ */

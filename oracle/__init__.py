@@ -1,0 +1,22 @@
+"""CPU oracle for the flash-decode hot path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the shipped package imports this directory.  Only the test-suite,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import it, and only as the checker -- never as the thing being measured or
+shipped.  The product path raises when its HIP library is missing; it never
+routes through this code.
+"""
+from .ref_decode import (  # noqa: F401
+    ref_paged_attn,
+    ref_paged_attn_lse,
+    fp8_e4m3fn_decode_table,
+    dequant_fp8_cache,
+    quantize_fp8_cache,
+)
+from .split_combine_model import (  # noqa: F401
+    split_range,
+    model_split_kv,
+    model_combine,
+    model_gqa_fwd_batch_decode,
+    model_sp_decode,
+)

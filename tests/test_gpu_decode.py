@@ -1,0 +1,386 @@
+"""GPU parity tests of the split-KV decode + combine path against the CPU oracle.
+
+Every test calls the HIP kernels through the C ABI (ctypes) via the package's
+reference-compatible wrappers and compares with ``oracle.ref_paged_attn_lse`` on
+the same seeded inputs.  Tolerances: the reference's own (atol = rtol = 1e-2,
+test_decode_attn.py:164) for its fp16 grid; the north-star gate (max-abs <= 2e-2 on
+16-bit outputs, <= 1e-3 relative on LSE) everywhere.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import DEV, assert_lse_close, assert_out_close, oracle_decode, run_decode
+
+pytestmark = pytest.mark.gpu
+
+NUM_BLOCKS = 4096  # pool pages of the grid tests (the 2^31-offset case has its own test)
+
+
+def _grid_workload(fd, kv_lens, num_heads, head_size, block_size, dtype, soft_cap, seed=0, num_blocks=NUM_BLOCKS):
+    """Inputs built the way test_decode_attn.py:140-156 builds them: N(0,1) q/k/v, block table
+    drawn with replacement, entries past ceil(kv_len/page) random as well."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    Hq, Hkv = num_heads
+    B = len(kv_lens)
+    q = torch.randn(B, Hq, head_size, generator=gen).to(dtype)
+    kv = torch.randn(num_blocks + 1, 2, block_size, Hkv, head_size, generator=gen).to(dtype)
+    k_cache = kv[:, 0].contiguous()
+    v_cache = kv[:, 1].contiguous()
+    max_blocks = (max(kv_lens) + block_size - 1) // block_size
+    bt = torch.randint(0, num_blocks, (B, max_blocks), generator=gen, dtype=torch.int32)
+    return fd.utils.DecodeWorkload(name="grid", q=q, k_cache=k_cache, v_cache=v_cache,
+                                   kv_lens=torch.tensor(kv_lens, dtype=torch.int32), block_table=bt,
+                                   scale=head_size ** -0.5, kv_split=32, soft_cap=float(soft_cap))
+
+
+# ---- the reference's own parameter grid (test_decode_attn.py:126-131)
+@pytest.mark.parametrize("kv_lens", [[1320, 18, 463], [1, 54, 293, 70]])
+@pytest.mark.parametrize("num_heads", [(16, 16), (32, 8), (64, 8), (6, 1)])
+@pytest.mark.parametrize("head_size", [128, 256])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("soft_cap", [0, 30, 50])
+def test_reference_grid_fp16(fd, kv_lens, num_heads, head_size, block_size, soft_cap):
+    wl = _grid_workload(fd, kv_lens, num_heads, head_size, block_size, torch.float16, soft_cap)
+    out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    torch.testing.assert_close(out.float(), ref, atol=1e-2, rtol=1e-2)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("num_heads", [(16, 16), (8, 4), (32, 8), (64, 8), (6, 1), (32, 2), (3, 1)])
+@pytest.mark.parametrize("block_size", [1, 16, 7])
+def test_other_dtypes_and_groups(fd, dtype, num_heads, block_size):
+    wl = _grid_workload(fd, [1320, 18, 463, 1, 70], num_heads, 128, block_size, dtype, 0, seed=3)
+    out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref, atol=2e-2 if dtype != torch.float32 else 2e-4)
+    assert_lse_close(lse, ref_lse, rtol=1e-3 if dtype != torch.float32 else 1e-5)
+
+
+@pytest.mark.parametrize("path", ["valu", "mfma"])
+@pytest.mark.parametrize("waves", [1, 2, 4, 8])
+def test_paths_and_waves_agree(fd, path, waves):
+    wl = _grid_workload(fd, [1320, 18, 463, 2049, 33], (32, 8), 128, 16, torch.bfloat16, 0, seed=5)
+    out, lse = run_decode(fd, wl, path=path, waves_per_block=waves)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+# ---- AOT (explicit stream) and persistent variants (test_decode_attn.py:168-251)
+@pytest.mark.parametrize("kv_len", [32, 1320, 18, 463, 1, 54, 293, 70])
+def test_aot_variant(fd, kv_len):
+    wl = _grid_workload(fd, [kv_len], (96, 12), 128, 1, torch.float16, 0, seed=kv_len).to(DEV)
+    stream = torch.cuda.current_stream()
+    for _ in range(10):
+        out = fd.gqa_fwd_batch_decode_aot(stream, wl.q, wl.k_cache, wl.v_cache, None, [1], wl.kv_lens,
+                                          wl.block_table, wl.scale, 0)
+    torch.cuda.synchronize()
+    ref, _ = oracle_decode(wl.to("cpu"))
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("kv_len", [1320, 18, 463, 1, 54, 293, 70])
+def test_persistent_variant(fd, kv_len):
+    wl = _grid_workload(fd, [kv_len], (64, 8), 128, 1, torch.float16, 0, seed=kv_len + 7)
+    out, lse = run_decode(fd, wl, variant="persistent")
+    ref, ref_lse = oracle_decode(wl)
+    torch.testing.assert_close(out.float(), ref, atol=1e-2, rtol=1e-2)
+    assert_lse_close(lse, ref_lse)
+
+
+def test_persistent_matches_plain_on_ragged_batch(fd):
+    wl = _grid_workload(fd, [70, 4000, 1, 900, 2500, 17], (32, 8), 128, 16, torch.bfloat16, 0, seed=11)
+    out_p, lse_p = run_decode(fd, wl, variant="persistent")
+    out, lse = run_decode(fd, wl)
+    assert torch.equal(out_p, out) and torch.equal(lse_p, lse)  # issue order must not change results
+
+
+# ---- the benchmark configurations
+@pytest.mark.parametrize("idx,scale_down", [(1, 1), (2, 8), (3, 16), (4, 8), (5, 16)])
+def test_configs_scaled(fd, idx, scale_down):
+    wl = fd.utils.make_config(idx, scale_down=scale_down)
+    kw = {}
+    if wl.extra_out is not None:
+        kw["extra_partials"] = (wl.extra_out.to(DEV), wl.extra_lse.to(DEV))
+    out, lse = run_decode(fd, wl, **kw)
+    ref, ref_lse = oracle_decode(wl)
+    if wl.extra_out is not None:
+        ref, ref_lse = _merge_extra(ref, ref_lse, wl.extra_out, wl.extra_lse)
+    fp32 = wl.q.dtype == torch.float32
+    assert_out_close(out, ref, atol=2e-4 if fp32 else 2e-2)
+    assert_lse_close(lse, ref_lse, rtol=1e-5 if fp32 else 1e-3)
+
+
+def _merge_extra(out, lse, extra_out, extra_lse):
+    """Closed form of the LSE merge: sum_r softmax(lse)_r * out_r, logsumexp(lse)."""
+    all_o = torch.cat([out[None].double(), extra_out.double()], 0)
+    all_l = torch.cat([lse[None].double(), extra_lse.double()], 0)
+    w = torch.softmax(all_l, dim=0)
+    return (w[..., None] * all_o).sum(0).float(), torch.logsumexp(all_l, 0).float()
+
+
+def test_config2_full_size(fd):
+    wl = fd.utils.make_config(2)
+    assert wl.algorithmic_bytes() == 268_583_968
+    out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+    # size-independent property: the result does not depend on the number of splits
+    wl.kv_split = 8
+    out8, lse8 = run_decode(fd, wl)
+    assert_out_close(out8, out.float(), atol=1e-2)
+    assert_lse_close(lse8, lse, rtol=1e-5)
+
+
+def test_config3_full_size_with_extra_partials(fd):
+    wl = fd.utils.make_config(3)
+    assert wl.algorithmic_bytes() == 536_978_436
+    out, lse = run_decode(fd, wl, extra_partials=(wl.extra_out.to(DEV), wl.extra_lse.to(DEV)))
+    ref, ref_lse = oracle_decode(wl)
+    ref, ref_lse = _merge_extra(ref, ref_lse, wl.extra_out, wl.extra_lse)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+def test_config4_full_size_sampled(fd):
+    wl = fd.utils.make_config(4)
+    out, lse = run_decode(fd, wl, variant="persistent")
+    rows = [0, 7, 21, 40, 63]  # the oracle checks a sample of the 64 sequences
+    ref, ref_lse = oracle_decode(wl, rows=rows)
+    assert_out_close(out[rows], ref)
+    assert_lse_close(lse[rows], ref_lse)
+    out2, lse2 = run_decode(fd, wl)   # unscheduled launch: identical bits
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
+def test_config5_full_size_sampled(fd):
+    wl = fd.utils.make_config(5)
+    out, lse = run_decode(fd, wl)
+    rows = [0, 13, 31]
+    ref, ref_lse = oracle_decode(wl, rows=rows)
+    assert_out_close(out[rows], ref)
+    assert_lse_close(lse[rows], ref_lse)
+
+
+# ---- edge cases
+def test_empty_and_short_sequences(fd):
+    """kv_len 0 (defined: out 0, lse -inf), kv_len < S (empty splits), kv_len == 1."""
+    wl = _grid_workload(fd, [0, 1, 5, 31, 32, 33, 64, 100], (32, 8), 128, 16, torch.bfloat16, 0, seed=21)
+    for variant in ("plain", "persistent"):
+        out, lse = run_decode(fd, wl, variant=variant)
+        ref, ref_lse = oracle_decode(wl)
+        assert torch.all(out[0] == 0) and torch.all(torch.isneginf(lse[0]))
+        assert_out_close(out, ref)
+        assert_lse_close(lse, ref_lse)
+
+
+def test_poisoned_pool_and_garbage_table(fd):
+    """Unreferenced pages hold NaN and table entries past ceil(kv_len/P) are out of range:
+    neither may influence the result (the reference leaves such entries random, test_decode_attn.py:156)."""
+    wl = _grid_workload(fd, [100, 37, 513], (32, 8), 128, 16, torch.bfloat16, 0, seed=23, num_blocks=256)
+    ref, ref_lse = oracle_decode(wl)
+    used = set()
+    for b, n in enumerate(wl.kv_lens.tolist()):
+        npg = -(-n // 16)
+        used.update(wl.block_table[b, :npg].tolist())
+        wl.block_table[b, npg:] = 2 ** 30  # far outside the pool
+    poison = torch.ones(wl.k_cache.shape[0], dtype=torch.bool)
+    poison[list(used)] = False
+    wl.k_cache[poison] = float("nan")
+    wl.v_cache[poison] = float("nan")
+    # the unused tail of the last page of every sequence is poisoned as well
+    for b, n in enumerate(wl.kv_lens.tolist()):
+        if n % 16:
+            page = int(wl.block_table[b, n // 16])
+            if sum(1 for bb, nn in enumerate(wl.kv_lens.tolist())
+                   if page in wl.block_table[bb, :-(-nn // 16)].tolist()) == 1:
+                wl.k_cache[page, n % 16:] = float("nan")
+                wl.v_cache[page, n % 16:] = float("nan")
+    for path in ("mfma", "valu"):
+        out, lse = run_decode(fd, wl, path=path)
+        assert_out_close(out, ref)
+        assert_lse_close(lse, ref_lse)
+
+
+def test_block_table_indexing_is_bit_exact(fd):
+    """Permuting the pool pages together with the table, and duplicating pages, leaves the output bits unchanged."""
+    wl = _grid_workload(fd, [777, 130], (32, 8), 128, 16, torch.bfloat16, 0, seed=25, num_blocks=128)
+    out, lse = run_decode(fd, wl)
+    gen = torch.Generator(device="cpu").manual_seed(99)
+    perm = torch.randperm(wl.k_cache.shape[0], generator=gen)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(perm.numel())
+    wl2 = fd.utils.DecodeWorkload(**{**wl.__dict__})
+    wl2.k_cache = wl.k_cache[perm].contiguous()
+    wl2.v_cache = wl.v_cache[perm].contiguous()
+    wl2.block_table = inv[wl.block_table.long()].to(torch.int32)
+    out2, lse2 = run_decode(fd, wl2)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
+def test_offsets_beyond_2_31_bytes(fd):
+    """A pool whose byte offsets exceed 2^31 (the reference computes them in int32, flash_decode.py:205-206)."""
+    Hkv, D, P = 8, 128, 16
+    pages = (2 ** 31) // (P * Hkv * D * 2) + 600       # > 2 GiB per cache
+    gen = torch.Generator(device="cpu").manual_seed(31)
+    k_cache = torch.empty(pages, P, Hkv, D, dtype=torch.bfloat16, device=DEV).normal_()
+    v_cache = torch.empty(pages, P, Hkv, D, dtype=torch.bfloat16, device=DEV).normal_()
+    kv_lens = [300, 129]
+    maxp = -(-max(kv_lens) // P)
+    bt = torch.randint(pages - 500, pages, (2, maxp), generator=gen, dtype=torch.int32)  # all in the high region
+    q = torch.randn(2, 32, D, generator=gen).to(torch.bfloat16)
+    lse = torch.empty(2, 32, dtype=torch.float32, device=DEV)
+    out = fd.gqa_fwd_batch_decode(q.to(DEV), k_cache, v_cache, None, [1, 1],
+                                  torch.tensor(kv_lens, dtype=torch.int32, device=DEV), bt.to(DEV), D ** -0.5,
+                                  lse_out=lse)
+    torch.cuda.synchronize()
+    # oracle on the referenced pages only, with the table remapped into the compact copy
+    used = torch.unique(bt.long())
+    remap = torch.zeros(pages, dtype=torch.long)
+    remap[used] = torch.arange(used.numel())
+    kc = k_cache[used.to(DEV)].cpu().float()
+    vc = v_cache[used.to(DEV)].cpu().float()
+    ref, ref_lse = oracle.ref_paged_attn_lse(q.float(), kc, vc, kv_lens, remap[bt.long()].to(torch.int32), D ** -0.5)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+def test_strided_inputs(fd):
+    """K and V as head-slices of one fused [pages, P, 2*Hkv, D] tensor and q as a slice of a wider
+    tensor: token / head / batch strides are honoured, nothing is copied."""
+    gen = torch.Generator(device="cpu").manual_seed(41)
+    fused = torch.randn(300, 16, 16, 128, generator=gen).to(torch.bfloat16)
+    qw = torch.randn(3, 32, 256, generator=gen).to(torch.bfloat16)
+    kv_lens = [500, 16, 1000]
+    bt = torch.randint(0, 300, (3, 63), generator=gen, dtype=torch.int32)
+    g_fused, g_q = fused.to(DEV), qw.to(DEV)
+    k, v = g_fused[:, :, :8], g_fused[:, :, 8:]
+    assert not k.is_contiguous() and not v.is_contiguous()
+    lse = torch.empty(3, 32, dtype=torch.float32, device=DEV)
+    out = fd.gqa_fwd_batch_decode(g_q[:, :, 128:], k, v, None, [1] * 3,
+                                  torch.tensor(kv_lens, dtype=torch.int32, device=DEV), bt.to(DEV), 128 ** -0.5,
+                                  lse_out=lse)
+    torch.cuda.synchronize()
+    ref, ref_lse = oracle.ref_paged_attn_lse(qw[:, :, 128:].float(), fused[:, :, :8].float(), fused[:, :, 8:].float(),
+                                             kv_lens, bt, 128 ** -0.5)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+# ---- caller-supplied partial buffers in the reference layout [B, Hq, S, Dv+1]
+@pytest.mark.parametrize("mid_dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("num_heads", [(32, 8), (4, 4)])
+def test_output_split_layout(fd, mid_dtype, num_heads):
+    wl = _grid_workload(fd, [1320, 18, 463], num_heads, 128, 16, torch.float16, 0, seed=51)
+    g = wl.to(DEV)
+    B, Hq, D = g.q.shape
+    S = 16
+    mid = torch.full((B, Hq, S, D + 1), 7.0, dtype=mid_dtype, device=DEV)
+    outc = torch.empty(B, Hq, D, dtype=torch.float16, device=DEV)
+    ret = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, [1] * B, g.kv_lens, g.block_table, g.scale, 0.0,
+                                  output_split=mid, output_combine=outc, kv_split=S)
+    torch.cuda.synchronize()
+    assert ret is outc                                   # the same object is returned (flash_decode.py:844)
+    model = oracle.model_split_kv(wl.q.float(), wl.k_cache.float(), wl.v_cache.float(), wl.kv_lens.tolist(),
+                                  wl.block_table, wl.scale, S)
+    got = mid.float().cpu()
+    loose = mid_dtype != torch.float32
+    # empty splits: out 0, lse -inf; others match the per-split model
+    assert torch.equal(torch.isneginf(got[..., D]), torch.isneginf(model[..., D]))
+    fin = ~torch.isneginf(model[..., D])
+    assert_out_close(got[..., :D][fin], model[..., :D][fin], atol=2e-2 if loose else 5e-3)
+    assert_lse_close(got[..., D][fin], model[..., D][fin], rtol=1e-2 if loose else 1e-3)
+    assert torch.all(got[..., :D][~fin] == 0)
+    ref, _ = oracle_decode(wl)
+    assert_out_close(outc, ref)
+
+
+def test_intra_rank_packs_lse_column(fd):
+    wl = _grid_workload(fd, [1320, 18, 463], (32, 8), 128, 16, torch.bfloat16, 0, seed=53)
+    g = wl.to(DEV)
+    outc = torch.empty(3, 32, 129, dtype=torch.float32, device=DEV)
+    fd.gqa_fwd_batch_decode_intra_rank(g.q, g.k_cache, g.v_cache, None, [1] * 3, g.kv_lens, g.block_table, g.scale,
+                                       output_combine=outc)
+    torch.cuda.synchronize()
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(outc[..., :128], ref)
+    assert_lse_close(outc[..., 128], ref_lse)
+
+
+# ---- fp8
+def test_fp8_dequant_table_through_the_kernel(fd):
+    """kv_len == 1 makes out == dequantised V[0]: all 256 byte patterns (NaN patterns excluded)
+    must come back as table[byte] * v_scale."""
+    tab = torch.from_numpy(oracle.fp8_e4m3fn_decode_table())
+    bytes_ = torch.arange(256, dtype=torch.uint8)
+    bytes_[0x7f] = 0
+    bytes_[0xff] = 0x80
+    Hkv, D = 2, 128
+    v = torch.zeros(2, 1, Hkv, D, dtype=torch.uint8)
+    v[0, 0, 0] = bytes_[:128]
+    v[0, 0, 1] = bytes_[128:]
+    v[1, 0, 0] = bytes_[128:]
+    v[1, 0, 1] = bytes_[:128]
+    k = torch.full_like(v, 0x38)  # 1.0
+    k_scale = torch.tensor([0.5, 2.0])
+    v_scale = torch.tensor([0.25, 3.0])
+    q = torch.ones(2, 8, D, dtype=torch.bfloat16)
+    bt = torch.tensor([[0], [1]], dtype=torch.int32)
+    for path in ("valu", "auto"):
+        lse = torch.empty(2, 8, dtype=torch.float32, device=DEV)
+        out = fd.gqa_fwd_batch_decode(q.to(DEV), k.to(DEV), v.to(DEV), None, [1, 1],
+                                      torch.tensor([1, 1], dtype=torch.int32, device=DEV), bt.to(DEV), 0.125,
+                                      output_combine=torch.empty(2, 8, D, dtype=torch.float32, device=DEV),
+                                      lse_out=lse, k_scale=k_scale.to(DEV), v_scale=v_scale.to(DEV), path=path)
+        torch.cuda.synchronize()
+        out = out.cpu()
+        for b in range(2):
+            for h in range(8):
+                kvh = h // 4
+                expect = tab[v[b, 0, kvh].long()] * v_scale[kvh]
+                assert torch.equal(out[b, h], expect), (path, b, h)
+                # one key: lse = scale * q.k = 0.125 * 128 * k_scale
+                assert math.isclose(lse[b, h].item(), 0.125 * 128 * k_scale[kvh].item(), rel_tol=1e-6)
+
+
+@pytest.mark.parametrize("num_heads", [(64, 8), (16, 4), (8, 8)])
+def test_fp8_decode_matches_oracle_on_dequantised_cache(fd, num_heads):
+    wl = fd.utils.make_paged_workload("fp8", [1000, 17, 4097], num_heads[0], num_heads[1], 128, 16, torch.bfloat16, 16,
+                                      seed=61, fp8_kv=True)
+    out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+
+
+# ---- scheduler
+def test_schedule_orders_longest_first(fd):
+    gen = torch.Generator(device="cpu").manual_seed(71)
+    for B in (1, 2, 64, 300, 1025):
+        lens = torch.randint(0, 50, (B,), generator=gen, dtype=torch.int32)
+        order = fd.schedule_sequences(lens.to(DEV)).cpu()
+        expect = torch.argsort(lens, descending=True, stable=True).to(torch.int32)
+        assert torch.equal(order, expect)
+
+
+# ---- error behaviour of the boundary
+def test_errors_are_reported_not_fatal(fd):
+    wl = _grid_workload(fd, [100], (32, 8), 128, 16, torch.float16, 0).to(DEV)
+    with pytest.raises(AssertionError):   # head-dim mismatch: the reference asserts too (flash_decode.py:767)
+        fd.gqa_fwd_batch_decode(wl.q[:, :, :64], wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0)
+    with pytest.raises(RuntimeError, match="MFMA path"):
+        fd.gqa_fwd_batch_decode(wl.q[:, :8], wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0,
+                                path="mfma")   # group 1 cannot take the MFMA path
+    with pytest.raises(RuntimeError, match="Unsupported data type"):
+        fd.gqa_fwd_batch_decode(wl.q.double(), wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0)
+    # and the library still works afterwards
+    out = fd.gqa_fwd_batch_decode(wl.q, wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, wl.scale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()

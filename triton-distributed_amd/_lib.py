@@ -1,0 +1,100 @@
+"""ctypes binding of libflash_decode_gfx950.so (the C ABI declared in include/flash_decode.h).
+
+The library is the only compute path of this package: if it is missing or a
+call fails, a ``RuntimeError`` is raised.  There is no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_void_p
+
+import torch
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libflash_decode_gfx950.so"
+LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
+
+FD_ABI_VERSION = 1
+
+# fd_dtype
+FD_F32, FD_F16, FD_BF16, FD_FP8_E4M3 = 0, 1, 2, 3
+# fd_path
+FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
+# fd_combine_mode
+FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
+
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_schedule", "fd_last_error", "fd_abi_version")
+
+_DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
+if hasattr(torch, "float8_e4m3fn"):
+    _DTYPES[torch.float8_e4m3fn] = FD_FP8_E4M3
+
+
+def fd_dtype_of(t: torch.Tensor, fp8_bytes: bool = False) -> int:
+    """fd_dtype enum of a tensor; a uint8 tensor is taken as e4m3fn bit patterns when ``fp8_bytes``."""
+    if fp8_bytes and t.dtype == torch.uint8:
+        return FD_FP8_E4M3
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"Unsupported data type: {t.dtype}") from None
+
+
+class FdParams(Structure):
+    """Mirror of ``struct fd_params``."""
+    _fields_ = [
+        ("q_heads", c_int32), ("kv_heads", c_int32), ("head_dim", c_int32), ("page_size", c_int32),
+        ("num_splits", c_int32), ("num_pages", c_int32), ("max_pages_per_seq", c_int32),
+        ("q_dtype", c_int32), ("kv_dtype", c_int32), ("mid_dtype", c_int32), ("out_dtype", c_int32),
+        ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
+        ("path", c_int32), ("waves_per_block", c_int32),
+    ]
+
+
+_lib = None
+
+
+def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
+    """Loads the shared library once and declares the argument types of every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{LIB_NAME} is not built ({path} missing). Build it with "
+            f"`python {os.path.join(PKG_DIR, 'build.py')}`; this package has no fallback path.")
+    lib = ctypes.CDLL(path)
+    i64 = c_int64
+    lib.fd_split_kv.restype = c_int32
+    lib.fd_split_kv.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int32,
+        i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, POINTER(FdParams)]
+    lib.fd_combine.restype = c_int32
+    lib.fd_combine.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
+        i64, i64, i64, i64, i64, c_int32, c_void_p, c_void_p, c_int32, POINTER(FdParams)]
+    lib.fd_schedule.restype = c_int32
+    lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]
+    lib.fd_last_error.restype = c_char_p
+    lib.fd_last_error.argtypes = []
+    lib.fd_abi_version.restype = c_int32
+    lib.fd_abi_version.argtypes = []
+    if lib.fd_abi_version() != FD_ABI_VERSION:
+        raise RuntimeError(f"{path}: ABI version {lib.fd_abi_version()} != expected {FD_ABI_VERSION}; rebuild")
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    """Raises RuntimeError with the library's message for a non-zero status."""
+    if status != 0:
+        msg = _lib.fd_last_error().decode("utf-8", "replace") if _lib is not None else ""
+        raise RuntimeError(f"flash_decode library error {status}: {msg}")
+
+
+def stream_handle(stream=None) -> int:
+    """hipStream_t of ``stream`` (a torch stream) or of the current torch stream."""
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return stream.cuda_stream

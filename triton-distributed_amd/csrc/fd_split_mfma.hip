@@ -1,0 +1,267 @@
+// Split-KV GQA paged decode on MFMA (gfx950), head_dim 128, 16-bit KV cache.
+//
+// Replaces kernel_gqa_fwd_batch_decode_split_kv
+// (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) for GQA groups
+// of at least 4 query heads per KV head.
+//
+// Decomposition: one workgroup per (sequence, split, KV head, block of <=16
+// query heads); its W waves take contiguous runs of 32-token tiles of the split
+// and are merged through LDS at the end.
+//
+// Per 32-token tile and wave (lane = 16*g + c):
+//   * 8 + 8 global_load_dwordx4: load i fetches, for every g, the full 256-byte
+//     K (and V) row of token tau(g,i) = 4g + (i&3) + 16(i>>2); the 16 lanes of a
+//     wave row read consecutive 16-byte chunks, so every load instruction covers
+//     four whole rows.  Row addresses come from one block-table lookup per
+//     token (lanes 0..31), broadcast with ds_bpermute.
+//   * K is staged row-major in LDS (row pitch 272 B: conflict-free 128-bit
+//     reads) and read back in the MFMA A layout: lane (g, m) <- K[token m][8
+//     dims of chunk 4*ks+g].   S^T[token][head] = K . Q^T on
+//     v_mfma_f32_16x16x32_bf16/f16 with Q as the B operand (heads padded to 16).
+//     The result leaves lane (g, c) with the scores of head c for tokens
+//     4g..4g+3 (+16): exactly the tokens whose V rows the lane holds.
+//   * Online softmax in registers (base-2 domain); the row maximum is reduced
+//     over the 4 wave rows with two bpermutes, the row sum stays per lane until
+//     the end.
+//   * V never touches LDS: the 8x8 16-bit blocks a lane holds are transposed
+//     with v_perm_b32 into the A operand of O^T[dim][head] += V^T . P^T, so the
+//     accumulator also lives in the "lane c = head c" layout and is rescaled
+//     without any cross-lane traffic.
+#include "fd_common.h"
+
+namespace {
+
+constexpr int kD = 128;
+constexpr int kTile = 32;         // tokens per tile
+constexpr int kKRow = 272;        // LDS pitch of a staged K row in bytes (256 + 16 pad)
+constexpr int kWaveLds = kTile * kKRow;  // 8704 B per wave, reused for the wave's partial result
+constexpr int kHB = 16;           // head slots per workgroup (MFMA N)
+static_assert(kWaveLds >= (kHB * kD + 2 * kHB) * 4, "partial result must fit in the K staging buffer");
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__bf16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+};
+template <>
+struct Mma<_Float16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                  0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+};
+
+template <typename T, bool SOFTCAP>
+__global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a) {
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int W = blockDim.x >> 6;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const WorkItem w = decode_work_item(a);
+  const int ntok = w.end - w.start;
+  const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
+  const int tpw = (ntiles + W - 1) / W;
+  const int t0 = wave * tpw;
+  const int t1 = min(t0 + tpw, ntiles);
+
+  const int head_in_group = w.hb * kHB + c;
+  const bool head_ok = head_in_group < a.G;
+  const int head = w.kvh * a.G + head_in_group;
+
+  // Q as the MFMA B operand: lane (g, c) holds Q[head c][32*ks + 8g .. +7].
+  u32x4 qop[4];
+  {
+    const char* qp = (const char*)a.q + ((int64_t)w.b * a.sq_b + (int64_t)head * a.sq_h) * 2;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qop[ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
+    }
+  }
+
+  const int32_t* bt_row = a.bt + (int64_t)w.b * a.sbt;
+  const char* kbase = (const char*)a.k + ((int64_t)w.kvh * a.sk_h) * 2 + c * 16;
+  const char* vbase = (const char*)a.v + ((int64_t)w.kvh * a.sv_h) * 2 + c * 16;
+  const int k_pitch = (int)(a.sk_t * 2);
+  const int v_pitch = (int)(a.sv_t * 2);
+  char* kb = smem + wave * kWaveLds;
+
+  float scale2 = a.sm_scale * FD_LOG2E;  // scores are kept in the base-2 domain
+  const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
+
+  // Row vector of tile t: lane (l & 31) holds the flat cache row of token start + 32t + (l & 31),
+  // tokens past the split end are clamped to the last valid token (their scores are masked).
+  auto tile_rows = [&](int t) -> int {
+    int n = w.start + t * kTile + (lane & 31);
+    n = min(n, w.end - 1);
+    return token_row(a, bt_row, n);
+  };
+
+  u32x4 kraw[8], vraw[8];
+  int rows[8];
+  auto fetch_rows = [&](int rv) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rows[i] = __shfl(rv, 4 * g + (i & 3) + 16 * (i >> 2));
+  };
+  auto issue_k = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) kraw[i] = *(const u32x4*)(kbase + (int64_t)rows[i] * k_pitch);
+  };
+  auto issue_v = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) vraw[i] = *(const u32x4*)(vbase + (int64_t)rows[i] * v_pitch);
+  };
+
+  float m = -INFINITY;  // running max of head c (identical in the 4 wave rows)
+  float l = 0.f;        // this lane's share of the running sum
+  f32x4 acc[8];         // acc[j][i] = O[head c][dim 32g + 8i + j]
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int rv_next = 0;
+  if (t0 < t1) {
+    fetch_rows(tile_rows(t0));
+    issue_k();
+    issue_v();
+    if (t0 + 1 < t1) rv_next = tile_rows(t0 + 1);
+  }
+
+  for (int t = t0; t < t1; ++t) {
+    const bool has_next = t + 1 < t1;
+    // ---- K tile -> LDS, then start fetching the next tile's K into the freed registers
+    wave_lds_fence();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
+      *(u32x4*)(kb + tau * kKRow + c * 16) = kraw[i];
+    }
+    wave_lds_fence();
+    if (has_next) {
+      fetch_rows(rv_next);
+      issue_k();
+      if (t + 2 < t1) rv_next = tile_rows(t + 2);
+    }
+    // ---- S^T = K . Q^T
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      u32x4 a0 = *(const u32x4*)(kb + c * kKRow + (4 * ks + g) * 16);
+      u32x4 a1 = *(const u32x4*)(kb + (16 + c) * kKRow + (4 * ks + g) * 16);
+      s0 = Mma<T>::run(a0, qop[ks], s0);
+      s1 = Mma<T>::run(a1, qop[ks], s1);
+    }
+    // ---- online softmax (head c, tokens tau(g, 0..7))
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = s0[i];
+      x[4 + i] = s1[i];
+    }
+    const int n0 = w.start + t * kTile;
+    const bool full = n0 + kTile <= w.end;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = x[i];
+      if (SOFTCAP) {
+        v = fd_softcap(v * a.sm_scale, a.soft_cap, inv_cap) * FD_LOG2E;
+      } else {
+        v *= scale2;
+      }
+      const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
+      x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
+    }
+    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx);  // finite: every tile holds at least one valid token
+    const float alpha = fd_exp2(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x[i] = fd_exp2(x[i] - m_new);
+      psum += x[i];
+    }
+    l = l * alpha + psum;
+    if (__any(m_new > m)) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+    }
+    m = m_new;
+    u32x4 pop;  // P^T as the B operand: element e <-> token tau(g, e)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pop[e] = Mma<T>::pack(x[2 * e], x[2 * e + 1]);
+
+    // ---- V: transpose the lane's 8 tokens x 8 dims block into 8 A operands
+    u32x4 vop[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        vop[j][e] = __builtin_amdgcn_perm(vraw[2 * e + 1][j >> 1], vraw[2 * e][j >> 1], sel);
+    }
+    if (has_next) issue_v();
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = Mma<T>::run(vop[j], pop, acc[j]);
+  }
+
+  // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  wave_lds_fence();
+  float* part = (float*)kb;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f32x4 lo = {acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
+    f32x4 hi = {acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
+    *(f32x4*)(part + c * kD + 32 * g + 8 * i) = lo;
+    *(f32x4*)(part + c * kD + 32 * g + 8 * i + 4) = hi;
+  }
+  if (g == 0) {
+    part[kHB * kD + c] = m;
+    part[kHB * kD + kHB + c] = l;
+  }
+  __syncthreads();
+  const int nheads = min(kHB, a.G - w.hb * kHB);
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, W, w, w.kvh * a.G + w.hb * kHB, nheads, 1.0f);
+}
+
+}  // namespace
+
+int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
+  const unsigned grid = (unsigned)a.batch * a.S * a.Hkv * a.nhb;
+  const unsigned block = 64u * waves;
+  const size_t lds = (size_t)waves * kWaveLds;
+  void (*kern)(const SplitArgs) = nullptr;
+  if (kv_dtype == FD_BF16) {
+    kern = soft_cap ? fd_split_mfma16_kernel<__bf16, true> : fd_split_mfma16_kernel<__bf16, false>;
+  } else if (kv_dtype == FD_F16) {
+    kern = soft_cap ? fd_split_mfma16_kernel<_Float16, true> : fd_split_mfma16_kernel<_Float16, false>;
+  } else {
+    return FD_ERR_UNSUPPORTED;
+  }
+  if (lds > 64 * 1024) {
+    // more than the default 64 KB of dynamic LDS per workgroup (gfx950 has 160 KB per CU)
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return FD_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(block), lds, stream, a);
+  return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
+}

@@ -1,0 +1,33 @@
+"""Flash-decode kernels: the names the reference exports for this path from
+``python/triton_dist/kernels/nvidia/__init__.py:32-35``."""
+from .flash_decode import (  # noqa: F401
+    gqa_fwd_batch_decode,
+    gqa_fwd_batch_decode_aot,
+    gqa_fwd_batch_decode_intra_rank,
+    gqa_fwd_batch_decode_intra_rank_aot,
+    gqa_fwd_batch_decode_persistent,
+    gqa_fwd_batch_decode_persistent_aot,
+    kernel_inter_rank_gqa_fwd_batch_decode_combine_kv,
+    inter_rank_combine,
+    schedule_sequences,
+    get_split_kv_algo_info,
+    get_combine_kv_algo_info,
+    get_triton_split_kv_algo_info,
+    get_triton_combine_kv_algo_info,
+)
+
+__all__ = [
+    "get_triton_combine_kv_algo_info",
+    "get_triton_split_kv_algo_info",
+    "get_combine_kv_algo_info",
+    "get_split_kv_algo_info",
+    "gqa_fwd_batch_decode_aot",
+    "gqa_fwd_batch_decode_intra_rank_aot",
+    "gqa_fwd_batch_decode_intra_rank",
+    "gqa_fwd_batch_decode_persistent_aot",
+    "gqa_fwd_batch_decode_persistent",
+    "gqa_fwd_batch_decode",
+    "kernel_inter_rank_gqa_fwd_batch_decode_combine_kv",
+    "inter_rank_combine",
+    "schedule_sequences",
+]

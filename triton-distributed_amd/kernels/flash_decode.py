@@ -1,0 +1,274 @@
+"""Host wrappers of the gfx950 flash-decode kernels.
+
+Same names, argument order and return values as the reference's
+``python/triton_dist/kernels/nvidia/flash_decode.py`` wrappers
+(``gqa_fwd_batch_decode`` :763-844, ``gqa_fwd_batch_decode_intra_rank`` :847-928,
+``gqa_fwd_batch_decode_persistent`` :931-1005 and the ``*_aot`` twins
+:1008-1161), so the reference's call sites work unchanged.  Every function
+enqueues hand-written HIP kernels through the C ABI in
+``include/flash_decode.h`` on the current (or given) torch stream and returns
+``output_combine``; nothing synchronises with the host.
+
+Keyword-only additions that the reference does not have (all default off):
+  lse_out         fp32 [B, Hq] tensor that receives the merged natural-log LSE
+  k_scale/v_scale fp32 [Hkv] dequantisation scales of an fp8-e4m3 KV cache
+  extra_partials  (out [E,B,Hq,Dv], lse [E,B,Hq] fp32): further partials merged by
+                  the combine, standing in for what other sequence-parallel ranks
+                  would contribute
+  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences
+  path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
+
+Differences from the reference, on purpose: when ``output_split`` is not
+supplied the partials are kept in fp32 with the LSE in its own fp32 buffer (the
+reference allocates fp16 ``[B,Hq,S,Dv+1]``, :783-784); the default
+``output_combine`` has the query's dtype (the reference hard-codes fp16, :785,
+which is the same thing for the fp16 inputs its tests use).
+"""
+from __future__ import annotations
+
+from ctypes import byref
+from typing import Optional
+
+import torch
+
+from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
+                    FdParams, check, fd_dtype_of, load_library, stream_handle)
+
+_PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
+DEFAULT_KV_SPLITS = 32  # flash_decode.py:779
+
+
+def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size, split_kv=32, soft_cap=0.0):
+    """Meta-parameters of the split kernel, the counterpart of ``get_triton_split_kv_algo_info``
+    (flash_decode.py:103-109): what the gfx950 kernels use instead of BLOCK_N/BLOCK_H/num_warps."""
+    group = q_heads // kv_heads
+    mfma = q_head_dim == 128 and group >= 4
+    return {
+        "kv_group_num": group, "q_head_num": q_heads, "NUM_KV_SPLITS": split_kv, "PAGE_SIZE": page_size,
+        "soft_cap": soft_cap, "K_DIM": q_head_dim, "V_DIM": v_head_dim,
+        "path": "mfma" if mfma else "valu", "TILE_N": 32 if mfma else None, "BLOCK_H": min(16, group) if mfma else
+        min(4, group), "wave_size": 64,
+    }
+
+
+get_triton_split_kv_algo_info = get_split_kv_algo_info  # reference name (kernels/nvidia/__init__.py:34)
+
+
+def get_combine_kv_algo_info(split_kv=32, v_head_dim=128, block_dv=512):
+    """Counterpart of ``get_triton_combine_kv_algo_info`` (flash_decode.py:281-285)."""
+    return {"NUM_KV_SPLITS": split_kv, "Lv": v_head_dim, "BLOCK_DV": block_dv, "wave_size": 64, "waves": 1}
+
+
+get_triton_combine_kv_algo_info = get_combine_kv_algo_info
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("flash-decode tensors must live on the GPU; this package has no CPU path")
+
+
+def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """Kernel (3): int32 [B] sequence order, longest kv_len first, computed on the device."""
+    _require_cuda(kv_lens)
+    lib = load_library()
+    assert kv_lens.dtype == torch.int32 and kv_lens.is_contiguous()
+    if out is None:
+        out = torch.empty_like(kv_lens)
+    check(lib.fd_schedule(stream_handle(stream), kv_lens.data_ptr(), kv_lens.numel(), out.data_ptr()))
+    return out
+
+
+def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
+                 waves_per_block) -> FdParams:
+    p = FdParams()
+    p.q_heads = q.shape[1]
+    p.kv_heads = k_cache.shape[2]
+    p.head_dim = q.shape[2]
+    p.page_size = k_cache.shape[1]
+    p.num_splits = kv_split
+    p.num_pages = k_cache.shape[0]
+    p.max_pages_per_seq = block_table.shape[1]
+    p.q_dtype = fd_dtype_of(q)
+    p.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
+    p.mid_dtype = mid_dtype
+    p.out_dtype = out_dtype
+    p.soft_cap = float(soft_cap or 0.0)
+    p.k_scale = k_scale.data_ptr() if k_scale is not None else None
+    p.v_scale = v_scale.data_ptr() if v_scale is not None else None
+    p.path = _PATHS[path]
+    p.waves_per_block = waves_per_block
+    return p
+
+
+def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
+            kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
+            stream=None, path="auto", waves_per_block=0):
+    batch, q_heads, q_head_dim = q.shape
+    _, page_size, kv_heads, k_head_dim = k_cache.shape
+    assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
+    v_head_dim = v_cache.shape[-1]
+    assert q_heads % kv_heads == 0
+    assert v_head_dim == k_head_dim, "the gfx950 kernels need equal K and V head dims"
+    _require_cuda(q, k_cache, v_cache, kv_lens, block_table, output_split, output_combine)
+    assert kv_lens.dtype == torch.int32 and block_table.dtype == torch.int32
+    assert q.stride(-1) == 1 and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+    # kv_loc = page * P + slot is a flat token index (flash_decode.py:205-206): the pool must be linear in it
+    assert k_cache.stride(0) == page_size * k_cache.stride(1) and v_cache.stride(0) == page_size * v_cache.stride(1)
+    if (k_scale is None) != (v_scale is None):
+        raise RuntimeError("k_scale and v_scale must be given together")
+    num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
+    lib = load_library()
+    hstream = stream_handle(stream)
+
+    lse_split = None
+    if output_split is None:
+        # internal partials: fp32, 128-bit aligned rows, LSE in its own buffer
+        n_o = batch * q_heads * num_splits * v_head_dim
+        n_l = batch * q_heads * num_splits
+        if (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
+                and workspace.is_contiguous() and workspace.numel() >= n_o + n_l):
+            # a float32 workspace that is large enough holds the partials: no allocation in the call
+            flat = workspace.view(-1)
+            output_split = flat[:n_o].view(batch, q_heads, num_splits, v_head_dim)
+            lse_split = flat[n_o:n_o + n_l].view(batch, q_heads, num_splits)
+        else:
+            output_split = torch.empty([batch, q_heads, num_splits, v_head_dim], dtype=torch.float32, device=q.device)
+            lse_split = torch.empty([batch, q_heads, num_splits], dtype=torch.float32, device=q.device)
+    else:
+        assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
+    out_cols = v_head_dim + 1 if with_lse_column else v_head_dim
+    if output_combine is None:
+        output_combine = torch.empty([batch, q_heads, out_cols], dtype=q.dtype, device=q.device)
+    else:
+        assert output_combine.shape[-1] >= out_cols and output_combine.stride(-1) == 1
+
+    p = _make_params(q, k_cache, block_table, num_splits, soft_cap, fd_dtype_of(output_split),
+                     fd_dtype_of(output_combine), k_scale, v_scale, path, waves_per_block)
+    check(lib.fd_split_kv(
+        hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_split.data_ptr(),
+        lse_split.data_ptr() if lse_split is not None else None, float(scale), block_table.data_ptr(),
+        kv_lens.data_ptr(), batch,
+        q.stride(0), q.stride(1), k_cache.stride(-3), k_cache.stride(-2), v_cache.stride(-3), v_cache.stride(-2),
+        output_split.stride(0), output_split.stride(1), output_split.stride(2), block_table.stride(0),
+        seq_order.data_ptr() if seq_order is not None else None, byref(p)))
+
+    ex_out = ex_lse = None
+    n_extra = 0
+    if extra_partials is not None:
+        ex_out, ex_lse = extra_partials
+        _require_cuda(ex_out, ex_lse)
+        n_extra = ex_out.shape[0]
+        assert tuple(ex_out.shape) == (n_extra, batch, q_heads, v_head_dim) and ex_out.is_contiguous()
+        assert tuple(ex_lse.shape) == (n_extra, batch, q_heads) and ex_lse.dtype == torch.float32
+        assert ex_lse.is_contiguous() and ex_out.dtype == output_combine.dtype
+    if lse_out is not None:
+        assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
+    check(lib.fd_combine(
+        hstream, output_split.data_ptr(), lse_split.data_ptr() if lse_split is not None else None,
+        output_combine.data_ptr(), lse_out.data_ptr() if lse_out is not None else None, kv_lens.data_ptr(),
+        batch, q_heads, num_splits,
+        output_split.stride(0), output_split.stride(1), output_split.stride(2),
+        output_combine.stride(0), output_combine.stride(1),
+        FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
+        ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra, byref(p)))
+    return output_combine
+
+
+def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
+                         output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Split-KV decode + plain combine -> ``output_combine [B, Hq, Dv]`` (flash_decode.py:763-844).
+
+    ``q_lens`` is accepted and ignored, as in the reference; so is ``workspace``, unless it is a
+    contiguous float32 GPU tensor of at least ``B*Hq*S*(Dv+1)`` elements, in which case the split
+    partials live in it instead of in freshly allocated memory.
+    """
+    return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
+                   with_lse_column=False, **kw)
+
+
+def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                    soft_cap=0.0, output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Split-KV decode + combine that also stores the merged LSE at column Dv:
+    ``output_combine [B, Hq, Dv+1]`` (flash_decode.py:847-928)."""
+    return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
+                   with_lse_column=True, **kw)
+
+
+def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0,
+                                    output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Scheduled variant (flash_decode.py:931-1005).  The reference fuses split and combine
+    behind a spinning grid barrier on a fixed 132-workgroup grid; here the device-side
+    scheduler orders the sequences longest first and the hardware dispatcher balances the
+    workgroups over the CUs, so no co-residency assumption is needed."""
+    if kw.get("seq_order") is None:
+        kw["seq_order"] = schedule_sequences(kv_lens, stream=kw.get("stream"))
+    return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
+                   with_lse_column=False, **kw)
+
+
+def gqa_fwd_batch_decode_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0,
+                             output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Explicit-stream twin of ``gqa_fwd_batch_decode`` (flash_decode.py:1008-1063).  The library
+    is always ahead-of-time compiled, so no environment switch is involved."""
+    return gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap,
+                                output_split, output_combine, kv_split, stream=stream, **kw)
+
+
+def gqa_fwd_batch_decode_intra_rank_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                        soft_cap=0, output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Explicit-stream twin of ``gqa_fwd_batch_decode_intra_rank`` (flash_decode.py:1066-1121)."""
+    return gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                           soft_cap, output_split, output_combine, kv_split, stream=stream, **kw)
+
+
+def gqa_fwd_batch_decode_persistent_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                        soft_cap=0, output_split=None, output_combine=None, kv_split=-1, **kw):
+    """Explicit-stream twin of ``gqa_fwd_batch_decode_persistent`` (flash_decode.py:1124-1161)."""
+    return gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                           soft_cap, output_split, output_combine, kv_split, stream=stream, **kw)
+
+
+def inter_rank_combine(all_ranks_out: torch.Tensor, final_out: torch.Tensor, global_kv_lens: torch.Tensor,
+                       lse_out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """Merges per-rank partials ``[R, B, Hq, Dv+1]`` (LSE at column Dv) into ``final_out [B, Hq, Dv]``;
+    rank r contributes to sequence b iff ``global_kv_lens[r, b] > 0`` (flash_decode.py:482-532)."""
+    R, batch, q_heads, d1 = all_ranks_out.shape
+    return _inter_rank_launch(all_ranks_out, final_out, global_kv_lens, batch, q_heads, all_ranks_out.stride(1),
+                              all_ranks_out.stride(2), all_ranks_out.stride(0), final_out.stride(0),
+                              final_out.stride(1), R, 512, d1 - 1, lse_out=lse_out, stream=stream)
+
+
+def _inter_rank_launch(Mid_O, o, B_Seqlens, batch, q_heads, stride_mid_ob, stride_mid_oh, stride_mid_os, stride_obs,
+                       stride_oh, NUM_KV_SPLITS, BLOCK_DV, Lv, lse_out=None, stream=None):
+    _require_cuda(Mid_O, o, B_Seqlens)
+    assert B_Seqlens.dtype == torch.int32 and B_Seqlens.is_contiguous()
+    assert Mid_O.stride(-1) == 1 and o.stride(-1) == 1
+    lib = load_library()
+    p = FdParams()
+    p.q_heads = q_heads
+    p.head_dim = Lv
+    p.mid_dtype = fd_dtype_of(Mid_O)
+    p.out_dtype = fd_dtype_of(o)
+    check(lib.fd_combine(
+        stream_handle(stream), Mid_O.data_ptr(), None, o.data_ptr(),
+        lse_out.data_ptr() if lse_out is not None else None, B_Seqlens.data_ptr(), batch, q_heads, NUM_KV_SPLITS,
+        stride_mid_ob, stride_mid_oh, stride_mid_os, stride_obs, stride_oh, FD_COMBINE_RANK, None, None, 0, byref(p)))
+    return o
+
+
+class _InterRankCombineKernel:
+    """Callable with the launch syntax of the reference's Triton kernel
+    ``kernel_inter_rank_gqa_fwd_batch_decode_combine_kv[grid](Mid_O, o, B_Seqlens, batch, q_heads,
+    stride_mid_ob, stride_mid_oh, stride_mid_os, stride_obs, stride_oh, NUM_KV_SPLITS, BLOCK_DV, Lv)``
+    (flash_decode.py:482-497; launched at layers/nvidia/sp_flash_decode_layer.py:173-183).
+    The grid and BLOCK_DV are accepted and ignored: the HIP launch derives its own."""
+
+    def __getitem__(self, grid):
+        return _inter_rank_launch
+
+    def __call__(self, *args, **kw):
+        return _inter_rank_launch(*args, **kw)
+
+
+kernel_inter_rank_gqa_fwd_batch_decode_combine_kv = _InterRankCombineKernel()
