@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--variant", default="plain", choices=["plain", "persistent"])
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
+    ap.add_argument("--fuse", action="store_true", help="fuse the combine into the tail of the split kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
@@ -81,7 +82,8 @@ def main():
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
     workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev)
     q_lens = [1] * B
-    kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=args.path, waves_per_block=args.waves)
+    kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=args.path, waves_per_block=args.waves,
+              fuse_combine=args.fuse)
     if wl.k_scale is not None:
         kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
     if wl.extra_out is not None:
@@ -165,7 +167,7 @@ def main():
         "config": {"workload": wl.name, "batch": B, "q_heads": Hq, "kv_heads": wl.k_cache.shape[2], "head_dim": D,
                    "page_size": wl.k_cache.shape[1], "kv_splits": S,
                    "kv_len_total": int(wl_cpu.kv_lens.sum()), "kv_pools_rotated": len(pools),
-                   "variant": args.variant, "path": args.path},
+                   "variant": args.variant, "path": args.path, "fused_combine": args.fuse},
         "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,

@@ -159,6 +159,35 @@ FD_API int fd_combine(void* stream, const void* mid_o, const float* mid_lse, voi
                const fd_params* params);
 
 /*
+ * One decode step: split-KV decode + combine.  Replaces the host wrappers
+ * gqa_fwd_batch_decode (flash_decode.py:763-844: the two launches at :788 and
+ * :826) and gqa_fwd_batch_decode_intra_rank (flash_decode.py:847-928) with
+ * combine_mode FD_COMBINE_SPLIT / FD_COMBINE_SPLIT_LSE.  Arguments as for
+ * fd_split_kv and fd_combine; out_split / lse_split are the partial workspace
+ * (written, and readable by the caller afterwards).
+ *
+ *  tickets   NULL: two launches (split kernel, then combine kernel).
+ *            Otherwise at least batch * q_heads int32, zero-initialised once by the
+ *            caller and not shared by calls that may run concurrently: the combine is
+ *            fused into the split kernel -- the workgroup that finishes a (sequence,
+ *            head block) last merges that group's partials -- which saves the second
+ *            launch.  The library leaves the counters at zero.  (The reference's fused
+ *            variant, flash_decode.py:587-760, instead spins on a grid barrier word in
+ *            `workspace` and needs all workgroups co-resident; nothing here waits.)
+ */
+FD_API int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_cache,
+              void* out_split, float* lse_split, void* out, float* lse_out, float sm_scale,
+              const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
+              int64_t stride_q_bs, int64_t stride_q_h,
+              int64_t stride_k_tok, int64_t stride_k_h,
+              int64_t stride_v_tok, int64_t stride_v_h,
+              int64_t stride_o_bs, int64_t stride_o_h, int64_t stride_o_split,
+              int64_t stride_table_bs, int64_t stride_obs, int64_t stride_oh,
+              const int32_t* seq_order, int32_t combine_mode,
+              const void* extra_out, const float* extra_lse, int32_t num_extra,
+              int32_t* tickets, const fd_params* params);
+
+/*
  * Kernel (3): work scheduler.  Writes seq_order[batch]: sequence indices sorted by
  * kv_len descending (ties by index), computed on the device from kv_lens, so that
  * fd_split_kv issues the longest sequences' workgroups first and the hardware

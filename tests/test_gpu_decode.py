@@ -64,9 +64,10 @@ def test_other_dtypes_and_groups(fd, dtype, num_heads, block_size):
 
 @pytest.mark.parametrize("path", ["valu", "mfma"])
 @pytest.mark.parametrize("waves", [1, 2, 4, 8])
-def test_paths_and_waves_agree(fd, path, waves):
+@pytest.mark.parametrize("fuse", [True, False])
+def test_paths_and_waves_agree(fd, path, waves, fuse):
     wl = _grid_workload(fd, [1320, 18, 463, 2049, 33], (32, 8), 128, 16, torch.bfloat16, 0, seed=5)
-    out, lse = run_decode(fd, wl, path=path, waves_per_block=waves)
+    out, lse = run_decode(fd, wl, path=path, waves_per_block=waves, fuse_combine=fuse)
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
@@ -101,11 +102,26 @@ def test_persistent_matches_plain_on_ragged_batch(fd):
     assert torch.equal(out_p, out) and torch.equal(lse_p, lse)  # issue order must not change results
 
 
+def test_fused_combine_leaves_tickets_clean_and_repeats(fd):
+    """The fused combine's ticket counters must be back at zero after every launch: ten calls in a
+    row on changing inputs all have to match the two-launch path."""
+    for i in range(10):
+        wl = _grid_workload(fd, [1320 - 97 * i, 18 + i, 463, 5 * i], (32, 8), 128, 16, torch.bfloat16, 0, seed=100 + i)
+        out_f, lse_f = run_decode(fd, wl, fuse_combine=True)
+        out_u, lse_u = run_decode(fd, wl, fuse_combine=False)
+        assert_out_close(out_f, out_u.float(), atol=1e-2)
+        assert_lse_close(lse_f, lse_u, rtol=1e-5)
+    fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
+    for t in fk._TICKETS.values():
+        assert int(t.abs().sum().item()) == 0
+
+
 # ---- the benchmark configurations
+@pytest.mark.parametrize("fuse", [True, False])
 @pytest.mark.parametrize("idx,scale_down", [(1, 1), (2, 8), (3, 16), (4, 8), (5, 16)])
-def test_configs_scaled(fd, idx, scale_down):
+def test_configs_scaled(fd, idx, scale_down, fuse):
     wl = fd.utils.make_config(idx, scale_down=scale_down)
-    kw = {}
+    kw = {"fuse_combine": fuse}
     if wl.extra_out is not None:
         kw["extra_partials"] = (wl.extra_out.to(DEV), wl.extra_lse.to(DEV))
     out, lse = run_decode(fd, wl, **kw)

@@ -24,7 +24,7 @@ FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_schedule", "fd_last_error", "fd_abi_version")
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_last_error", "fd_abi_version")
 
 _DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
 if hasattr(torch, "float8_e4m3fn"):
@@ -55,11 +55,15 @@ class FdParams(Structure):
 _lib = None
 
 
-def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
-    """Loads the shared library once and declares the argument types of every entry point."""
+def load_library(path: str = None) -> ctypes.CDLL:
+    """Loads the shared library once and declares the argument types of every entry point.
+
+    ``FD_LIBRARY_PATH`` in the environment names another build of the library (same ABI)."""
     global _lib
     if _lib is not None:
         return _lib
+    if path is None:
+        path = os.environ.get("FD_LIBRARY_PATH", LIB_PATH)
     if not os.path.exists(path):
         raise RuntimeError(
             f"{LIB_NAME} is not built ({path} missing). Build it with "
@@ -74,6 +78,11 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.fd_combine.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
         i64, i64, i64, i64, i64, c_int32, c_void_p, c_void_p, c_int32, POINTER(FdParams)]
+    lib.fd_decode.restype = c_int32
+    lib.fd_decode.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+        c_int32, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p,
+        c_int32, c_void_p, POINTER(FdParams)]
     lib.fd_schedule.restype = c_int32
     lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]
     lib.fd_last_error.restype = c_char_p

@@ -32,11 +32,14 @@ int dtype_size(int dt) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int ilog2_exact(int x) {
-  if (x <= 0 || (x & (x - 1))) return -1;
-  int r = 0;
-  while ((1 << r) < x) ++r;
-  return r;
+// Magic number for n / d, exact for 0 <= n < 2^31: with l = ceil(log2 d) and k = 31 + l,
+// M = floor(2^k / d) + 1 fits in 32 bits and floor(n * M / 2^k) == floor(n / d).
+void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
+  uint32_t l = 0;
+  while (((uint64_t)1 << l) < d) ++l;
+  const uint32_t k = 31 + l;
+  *magic = (uint32_t)((((uint64_t)1 << k) / d) + 1);
+  *shift = k;
 }
 
 // Waves per workgroup when the caller does not choose: enough waves to put
@@ -57,46 +60,64 @@ int choose_waves(int64_t workgroups, int64_t max_tokens_per_split, int tile) {
 }  // namespace
 
 extern "C" {
-
 const char* fd_last_error(void) { return g_err; }
-
 int fd_abi_version(void) { return FD_ABI_VERSION; }
+}
 
-int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out_split,
-                float* lse_split, float sm_scale, const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
-                int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok, int64_t stride_k_h,
-                int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
-                int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p) {
-  if (!p) return fail(FD_ERR_INVALID_ARG, "fd_split_kv: params is NULL");
+namespace {
+
+struct FusedTail {          // what the fused combine needs on top of the split arguments
+  int32_t* tickets = nullptr;
+  void* out = nullptr;
+  float* lse_out = nullptr;
+  const void* extra_out = nullptr;
+  const float* extra_lse = nullptr;
+  int64_t stride_obs = 0, stride_oh = 0;
+  int32_t num_extra = 0, lse_column = 0;
+};
+
+// Largest dynamic LDS a workgroup may ask for on gfx950 (160 KB per CU).
+constexpr size_t kMaxLds = 160 * 1024;
+
+int split_impl(const char* fn, void* stream, const void* q, const void* k_cache, const void* v_cache,
+               void* out_split, float* lse_split, float sm_scale, const int32_t* block_table,
+               const int32_t* kv_lens, int32_t batch, int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok,
+               int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
+               int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p,
+               const FusedTail* tail, bool* fused) {
+  if (fused) *fused = false;
+  if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (!q || !k_cache || !v_cache || !out_split || !block_table || !kv_lens)
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: NULL tensor pointer");
-  if (batch < 0) return fail(FD_ERR_INVALID_ARG, "fd_split_kv: batch = %d", batch);
+    return fail(FD_ERR_INVALID_ARG, "%s: NULL tensor pointer", fn);
+  if (batch < 0) return fail(FD_ERR_INVALID_ARG, "%s: batch = %d", fn, batch);
   if (batch == 0) return FD_OK;
+  if (batch > 65535) return fail(FD_ERR_TOO_LARGE, "%s: batch %d > 65535 (grid z)", fn, batch);
   if (p->q_heads <= 0 || p->kv_heads <= 0 || p->q_heads % p->kv_heads != 0)
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: q_heads %d must be a positive multiple of kv_heads %d", p->q_heads,
+    return fail(FD_ERR_INVALID_ARG, "%s: q_heads %d must be a positive multiple of kv_heads %d", fn, p->q_heads,
                 p->kv_heads);
   if (p->page_size <= 0 || p->num_splits <= 0 || p->num_pages <= 0 || p->max_pages_per_seq <= 0)
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: page_size/num_splits/num_pages/max_pages_per_seq must be > 0");
+    return fail(FD_ERR_INVALID_ARG, "%s: page_size/num_splits/num_pages/max_pages_per_seq must be > 0", fn);
+  if (p->num_splits > 65535) return fail(FD_ERR_TOO_LARGE, "%s: num_splits %d > 65535 (grid y)", fn, p->num_splits);
   if ((int64_t)p->num_pages * p->page_size >= (int64_t)1 << 31)
-    return fail(FD_ERR_TOO_LARGE, "fd_split_kv: pool of %lld token rows exceeds 2^31",
+    return fail(FD_ERR_TOO_LARGE, "%s: pool of %lld token rows exceeds 2^31", fn,
                 (long long)p->num_pages * p->page_size);
-  if ((int64_t)p->max_pages_per_seq * p->page_size >= (int64_t)1 << 31)
-    return fail(FD_ERR_TOO_LARGE, "fd_split_kv: block table capacity exceeds 2^31 tokens");
+  if ((int64_t)p->max_pages_per_seq * p->page_size + p->num_splits >= (int64_t)1 << 31)
+    return fail(FD_ERR_TOO_LARGE, "%s: block table capacity exceeds 2^31 tokens", fn);
   const int D = p->head_dim;
-  if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "fd_split_kv: head_dim %d (64/128/256)", D);
+  if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "%s: head_dim %d (64/128/256)", fn, D);
   const int qsz = dtype_size(p->q_dtype), kvsz = dtype_size(p->kv_dtype), msz = dtype_size(p->mid_dtype);
-  if (!qsz || p->q_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "fd_split_kv: q_dtype %d", p->q_dtype);
-  if (!kvsz) return fail(FD_ERR_UNSUPPORTED, "fd_split_kv: kv_dtype %d", p->kv_dtype);
-  if (!msz || p->mid_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "fd_split_kv: mid_dtype %d", p->mid_dtype);
+  if (!qsz || p->q_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: q_dtype %d", fn, p->q_dtype);
+  if (!kvsz) return fail(FD_ERR_UNSUPPORTED, "%s: kv_dtype %d", fn, p->kv_dtype);
+  if (!msz || p->mid_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: mid_dtype %d", fn, p->mid_dtype);
   if (p->kv_dtype == FD_FP8_E4M3 && (!p->k_scale || !p->v_scale))
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: fp8 KV cache needs k_scale and v_scale");
+    return fail(FD_ERR_INVALID_ARG, "%s: fp8 KV cache needs k_scale and v_scale", fn);
   const int kv_elems16 = 16 / kvsz;
   if (!aligned16(k_cache) || !aligned16(v_cache) || stride_k_tok % kv_elems16 || stride_k_h % kv_elems16 ||
       stride_v_tok % kv_elems16 || stride_v_h % kv_elems16)
-    return fail(FD_ERR_ALIGNMENT, "fd_split_kv: K/V rows must be 16-byte aligned (pointer and token/head strides)");
+    return fail(FD_ERR_ALIGNMENT, "%s: K/V rows must be 16-byte aligned (pointer and token/head strides)", fn);
   if (stride_k_tok <= 0 || stride_v_tok <= 0 || stride_k_tok * kvsz >= ((int64_t)1 << 31) ||
       stride_v_tok * kvsz >= ((int64_t)1 << 31))
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: token stride out of range");
+    return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
   const int G = p->q_heads / p->kv_heads;
   const int64_t max_tok_split = ((int64_t)p->max_pages_per_seq * p->page_size + p->num_splits - 1) / p->num_splits;
 
@@ -110,7 +131,8 @@ int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_
   a.sbt = stride_table_bs;
   a.sm_scale = sm_scale; a.soft_cap = p->soft_cap > 0.f ? p->soft_cap : 0.f;
   a.batch = batch; a.Hq = p->q_heads; a.Hkv = p->kv_heads; a.G = G; a.S = p->num_splits; a.P = p->page_size;
-  a.log2P = ilog2_exact(p->page_size);
+  div_magic((uint32_t)p->page_size, &a.div_magic, &a.div_shift);
+  div_magic((uint32_t)p->num_splits, &a.s_magic, &a.s_shift);
   a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
   a.q_dtype = p->q_dtype; a.mid_dtype = p->mid_dtype;
   a.vec_out = (p->mid_dtype == FD_F32 && aligned16(out_split) && stride_o_bs % 4 == 0 && stride_o_h % 4 == 0 &&
@@ -123,33 +145,87 @@ int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "fd_split_kv: MFMA path needs head_dim 128, group >= 4 (<= 16 or a multiple of 16), 16-bit KV of the "
-                "query's dtype and 16-byte aligned q rows");
+                "%s: MFMA path needs head_dim 128, group >= 4 (<= 16 or a multiple of 16), 16-bit KV of the "
+                "query's dtype and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
-    return fail(FD_ERR_INVALID_ARG, "fd_split_kv: waves_per_block %d (0, 1, 2, 4 or 8)", p->waves_per_block);
+    return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
 
-  int rc;
+  int tile;
   if (use_mfma) {
     a.hbsz = G < 16 ? G : 16;
     a.nhb = (G + 15) / 16;
-    const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
-    if (wgs >= ((int64_t)1 << 31)) return fail(FD_ERR_TOO_LARGE, "fd_split_kv: %lld workgroups", (long long)wgs);
-    const int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, 32);
-    rc = fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);
+    tile = 32;
   } else {
-    a.hbsz = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
-    if (G == 3) a.hbsz = 4;
+    a.hbsz = G >= 3 ? 4 : G;
     a.nhb = (G + a.hbsz - 1) / a.hbsz;
-    const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
-    if (wgs >= ((int64_t)1 << 31)) return fail(FD_ERR_TOO_LARGE, "fd_split_kv: %lld workgroups", (long long)wgs);
-    const int tile = 4 * (64 / (D * kvsz / 16));
-    const int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
-    rc = fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, waves);
+    tile = 4 * (64 / (D * kvsz / 16));
   }
-  if (rc == FD_ERR_LAUNCH) return fail(rc, "fd_split_kv: launch failed: %s", hipGetErrorString(hipGetLastError()));
-  if (rc != FD_OK) return fail(rc, "fd_split_kv: no kernel for kv_dtype %d, head_dim %d, group %d", p->kv_dtype, D, G);
+  if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
+    return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
+  const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
+  const int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
+
+  // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS
+  if (tail && tail->tickets && p->mid_dtype == FD_F32) {  // the fused tail exchanges fp32 partials only
+    const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (use_mfma ? 16 : a.hbsz) * 4;
+    if (lse_lds <= kMaxLds / 2) {
+      a.tickets = tail->tickets; a.fout = tail->out; a.flse = tail->lse_out;
+      a.extra_out = tail->extra_out; a.extra_lse = tail->extra_lse;
+      a.sfo_b = tail->stride_obs; a.sfo_h = tail->stride_oh;
+      a.out_dtype = p->out_dtype; a.num_extra = tail->num_extra; a.lse_column = tail->lse_column;
+      if (fused) *fused = true;
+    }
+  }
+
+  int rc = use_mfma ? fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f)
+                    : fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, waves);
+  if (rc == FD_ERR_LAUNCH) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
+  if (rc != FD_OK) return fail(rc, "%s: no kernel for kv_dtype %d, head_dim %d, group %d", fn, p->kv_dtype, D, G);
   return FD_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out_split,
+                float* lse_split, float sm_scale, const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
+                int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok, int64_t stride_k_h,
+                int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
+                int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p) {
+  return split_impl("fd_split_kv", stream, q, k_cache, v_cache, out_split, lse_split, sm_scale, block_table, kv_lens,
+                    batch, stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_o_bs,
+                    stride_o_h, stride_o_split, stride_table_bs, seq_order, p, nullptr, nullptr);
+}
+
+int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out_split,
+              float* lse_split, void* out, float* lse_out, float sm_scale, const int32_t* block_table,
+              const int32_t* kv_lens, int32_t batch, int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok,
+              int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
+              int64_t stride_o_split, int64_t stride_table_bs, int64_t stride_obs, int64_t stride_oh,
+              const int32_t* seq_order, int32_t combine_mode, const void* extra_out, const float* extra_lse,
+              int32_t num_extra, int32_t* tickets, const fd_params* p) {
+  if (!out) return fail(FD_ERR_INVALID_ARG, "fd_decode: out is NULL");
+  if (combine_mode != FD_COMBINE_SPLIT && combine_mode != FD_COMBINE_SPLIT_LSE)
+    return fail(FD_ERR_INVALID_ARG, "fd_decode: combine_mode %d (FD_COMBINE_SPLIT or FD_COMBINE_SPLIT_LSE)",
+                combine_mode);
+  if (num_extra < 0 || (num_extra > 0 && (!extra_out || !extra_lse)))
+    return fail(FD_ERR_INVALID_ARG, "fd_decode: num_extra %d needs extra_out and extra_lse", num_extra);
+  if (p && (!dtype_size(p->out_dtype) || p->out_dtype == FD_FP8_E4M3))
+    return fail(FD_ERR_UNSUPPORTED, "fd_decode: out_dtype %d", p->out_dtype);
+  FusedTail tail;
+  tail.tickets = tickets; tail.out = out; tail.lse_out = lse_out; tail.extra_out = extra_out;
+  tail.extra_lse = extra_lse; tail.stride_obs = stride_obs; tail.stride_oh = stride_oh; tail.num_extra = num_extra;
+  tail.lse_column = combine_mode == FD_COMBINE_SPLIT_LSE;
+  bool fused = false;
+  int rc = split_impl("fd_decode", stream, q, k_cache, v_cache, out_split, lse_split, sm_scale, block_table, kv_lens,
+                      batch, stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_o_bs,
+                      stride_o_h, stride_o_split, stride_table_bs, seq_order, p, &tail, &fused);
+  if (rc != FD_OK || fused || batch == 0) return rc;
+  return fd_combine(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
+                    stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out, extra_lse,
+                    num_extra, p);
 }
 
 int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
@@ -166,7 +242,8 @@ int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out,
     return fail(FD_ERR_INVALID_ARG, "fd_combine: mode %d", mode);
   if (num_extra > 0 && (!extra_out || !extra_lse))
     return fail(FD_ERR_INVALID_ARG, "fd_combine: num_extra > 0 needs extra_out and extra_lse");
-  if (p->head_dim <= 0 || p->head_dim > 256) return fail(FD_ERR_UNSUPPORTED, "fd_combine: head_dim %d", p->head_dim);
+  if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)
+    return fail(FD_ERR_UNSUPPORTED, "fd_combine: head_dim %d (64/128/256)", p->head_dim);
   if (!dtype_size(p->mid_dtype) || p->mid_dtype == FD_FP8_E4M3 || !dtype_size(p->out_dtype) ||
       p->out_dtype == FD_FP8_E4M3)
     return fail(FD_ERR_UNSUPPORTED, "fd_combine: mid_dtype %d / out_dtype %d", p->mid_dtype, p->out_dtype);
@@ -178,6 +255,8 @@ int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out,
   a.s_mb = stride_mid_ob; a.s_mh = stride_mid_oh; a.s_ms = stride_mid_os; a.s_ob = stride_obs; a.s_oh = stride_oh;
   a.batch = batch; a.Hq = q_heads; a.D = p->head_dim; a.num_partials = num_partials; a.num_extra = num_extra;
   a.mode = mode; a.mid_dtype = p->mid_dtype; a.out_dtype = p->out_dtype;
+  a.vec_mid = (p->mid_dtype == FD_F32 && aligned16(mid_o) && stride_mid_ob % 4 == 0 && stride_mid_oh % 4 == 0 &&
+               stride_mid_os % 4 == 0) ? 1 : 0;
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;

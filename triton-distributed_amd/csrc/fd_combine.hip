@@ -3,35 +3,34 @@
 // fd_combine_kernel replaces the reference's three combine kernels
 // (python/triton_dist/kernels/nvidia/flash_decode.py:308-360 plain, :393-449
 // intra-rank with merged LSE, :482-532 inter-rank).  The reference walks the
-// partials sequentially with a running max; here one wave per (sequence, head)
-// first reduces the LSEs (max, then sum of weights) and then accumulates
-// sum_s w_s * O_s with all row loads independent of each other -- the same
-// value, out = sum_s softmax(LSE)_s * O_s and LSE = logsumexp_s(LSE_s), with two
-// dependent memory round trips instead of S.
+// partials sequentially with a running max.  Here one 256-thread workgroup per
+// (sequence, head) first brings all partial LSEs into LDS (one load per
+// thread), every thread derives M = max and the weights w_s = e^{LSE_s - M}
+// from there, and then the threads -- laid out as ROWS row groups x D/4
+// column groups -- accumulate sum_s w_s * O_s with 128-bit loads that do not
+// depend on each other.  The row groups are summed through LDS.  The value is
+// the reference's: out = sum_s softmax(LSE)_s * O_s, LSE = logsumexp_s(LSE_s);
+// the cost is two dependent memory round trips instead of S.
 #include "fd_common.h"
 
 namespace {
 
-constexpr int kMaxDPerLane = 4;  // head_dim <= 256
+constexpr int kCombineThreads = 256;
+constexpr int kMaxPartials = 1024;  // LSEs staged in LDS per pass
 
-__device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
-  return x;
-}
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o);
-  return x;
-}
+template <int D>
+__global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const CombineArgs a) {
+  constexpr int CG = D / 4;                    // column groups (one 128-bit chunk of fp32 each)
+  constexpr int ROWS = kCombineThreads / CG;   // partial rows in flight per pass
+  __shared__ float s_lse[kMaxPartials];
+  __shared__ __align__(16) float s_acc[ROWS][D];
+  __shared__ float s_l[ROWS];
 
-__global__ void __launch_bounds__(64) fd_combine_kernel(const CombineArgs a) {
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
   const int b = blockIdx.x / a.Hq;
   const int h = blockIdx.x - b * a.Hq;
   const int S = a.num_partials;
   const int NP = S + a.num_extra;
-  const int D = a.D;
   const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
 
   int kv_len = 0, per = 0;
@@ -39,69 +38,78 @@ __global__ void __launch_bounds__(64) fd_combine_kernel(const CombineArgs a) {
     kv_len = max(a.seqlens[b], 0);
     per = (kv_len + S - 1) / S;
   }
-  auto partial_valid = [&](int s) -> bool {
-    if (s >= S) return true;                                   // extra partials are always valid
-    if (a.mode == FD_COMBINE_RANK) return a.seqlens[(int64_t)s * a.batch + b] > 0;
-    int64_t st = (int64_t)per * s;                             // split range non-empty
-    return st < kv_len;
-  };
+  // LSE of partial s, -inf when the partial is not valid
   auto partial_lse = [&](int s) -> float {
-    if (s >= S) return a.extra_lse[((int64_t)(s - S) * a.batch + b) * a.Hq + h];
+    if (s >= S) return a.extra_lse[((int64_t)(s - S) * a.batch + b) * a.Hq + h];  // extras: always valid
+    if (a.mode == FD_COMBINE_RANK) {
+      if (a.seqlens[(int64_t)s * a.batch + b] <= 0) return -INFINITY;
+    } else if ((int64_t)per * s >= kv_len) {  // empty split range
+      return -INFINITY;
+    }
     if (a.mid_lse) return a.mid_lse[((int64_t)b * a.Hq + h) * S + s];
     return load_as_f32(a.mid_o, mid_base + (int64_t)s * a.s_ms + D, a.mid_dtype);
   };
 
-  // pass 1: M = max LSE over valid partials
-  float M = -INFINITY;
-  for (int s0 = 0; s0 < NP; s0 += 64) {
-    const int s = s0 + lane;
-    float L = -INFINITY;
-    if (s < NP && partial_valid(s)) L = partial_lse(s);
-    M = fmaxf(M, L);
-  }
-  M = wave_max(M);
+  const int r = tid / CG;
+  const int c = tid - r * CG;
+  const bool vec_mid = a.mid_dtype == FD_F32 && a.vec_mid;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float M = -INFINITY;  // running max over the passes (one pass unless NP > kMaxPartials)
+  float L = 0.f;        // sum of the weights of this thread's rows
 
-  float acc[kMaxDPerLane] = {0.f, 0.f, 0.f, 0.f};
-  float Lsum = 0.f;
-  if (M > -INFINITY) {
-    for (int s0 = 0; s0 < NP; s0 += 64) {
-      const int s = s0 + lane;
-      float wgt = 0.f;
-      if (s < NP && partial_valid(s)) wgt = __expf(partial_lse(s) - M);
-      Lsum += wgt;
-      const int cnt = min(64, NP - s0);
-      for (int j = 0; j < cnt; ++j) {
-        const float wj = __shfl(wgt, j);
-        if (wj == 0.f) continue;  // wave-uniform
-        const int sj = s0 + j;
+  for (int p0 = 0; p0 < NP; p0 += kMaxPartials) {
+    const int cnt = min(kMaxPartials, NP - p0);
+    __syncthreads();
+    for (int i = tid; i < cnt; i += kCombineThreads) s_lse[i] = partial_lse(p0 + i);
+    __syncthreads();
+    float m_pass = -INFINITY;
+    for (int i = 0; i < cnt; ++i) m_pass = fmaxf(m_pass, s_lse[i]);
+    const float m_new = fmaxf(M, m_pass);
+    if (m_new == -INFINITY) continue;  // nothing valid so far (uniform)
+    const float resc = __expf(M - m_new);  // 0 on the first valid pass
+    acc *= resc;
+    L *= resc;
+    M = m_new;
+    for (int i = r; i < cnt; i += ROWS) {
+      const float wgt = __expf(s_lse[i] - M);
+      if (wgt == 0.f) continue;
+      const int s = p0 + i;
+      f32x4 o;
+      if (s < S) {
+        const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
+        if (vec_mid) {
+          o = *(const f32x4*)((const float*)a.mid_o + off);
+        } else {
 #pragma unroll
-        for (int k = 0; k < kMaxDPerLane; ++k) {
-          const int d = lane + 64 * k;
-          if (d < D) {
-            float o;
-            if (sj < S) {
-              o = load_as_f32(a.mid_o, mid_base + (int64_t)sj * a.s_ms + d, a.mid_dtype);
-            } else {
-              o = load_as_f32(a.extra_out, (((int64_t)(sj - S) * a.batch + b) * a.Hq + h) * D + d, a.out_dtype);
-            }
-            acc[k] = fmaf(wj, o, acc[k]);
-          }
+          for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.mid_o, off + k, a.mid_dtype);
         }
-      }
-    }
-    Lsum = wave_sum(Lsum);
-  }
-  const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
-  const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
+      } else {
+        const int64_t off = (((int64_t)(s - S) * a.batch + b) * a.Hq + h) * D + 4 * c;
 #pragma unroll
-  for (int k = 0; k < kMaxDPerLane; ++k) {
-    const int d = lane + 64 * k;
-    if (d < D) store_from_f32(a.out, out_base + d, a.out_dtype, acc[k] * inv);
+        for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.extra_out, off + k, a.out_dtype);
+      }
+      acc += o * wgt;
+      L += wgt;
+    }
   }
-  if (lane == 0) {
-    const float lse = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
-    if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, lse);
-    if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = lse;
+  *(f32x4*)&s_acc[r][4 * c] = acc;
+  if (c == 0) s_l[r] = L;
+  __syncthreads();
+  if (tid < D) {
+    float o = 0.f, Lsum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      o += s_acc[i][tid];
+      Lsum += s_l[i];
+    }
+    const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+    const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
+    store_from_f32(a.out, out_base + tid, a.out_dtype, o * inv);
+    if (tid == 0) {
+      const float lse = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
+      if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, lse);
+      if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = lse;
+    }
   }
 }
 
@@ -123,7 +131,14 @@ __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restr
 
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a) {
   const unsigned grid = (unsigned)a.batch * a.Hq;
-  hipLaunchKernelGGL(fd_combine_kernel, dim3(grid), dim3(64), 0, stream, a);
+  void (*kern)(const CombineArgs) = nullptr;
+  switch (a.D) {
+    case 64: kern = fd_combine_kernel<64>; break;
+    case 128: kern = fd_combine_kernel<128>; break;
+    case 256: kern = fd_combine_kernel<256>; break;
+    default: return FD_ERR_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }
 

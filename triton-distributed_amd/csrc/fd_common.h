@@ -36,11 +36,22 @@ struct SplitArgs {
   const float* v_scale;
   int64_t sq_b, sq_h, sk_t, sk_h, sv_t, sv_h, so_b, so_h, so_s, sbt;
   float sm_scale, soft_cap;
-  int32_t batch, Hq, Hkv, G, S, P, log2P, max_pages, num_pages;
+  int32_t batch, Hq, Hkv, G, S, P, max_pages, num_pages;
+  uint32_t div_magic, div_shift;  // n / P == (uint64(n) * div_magic) >> div_shift for 0 <= n < 2^31
   int32_t q_dtype, mid_dtype;
   int32_t nhb;      // head blocks per KV head
   int32_t hbsz;     // query heads per head block
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
+  uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
+  // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
+  // merges its S partials (+ num_extra further ones) into the final output.
+  int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
+  void* fout;            // [batch, Hq, D(+1)] out_dtype
+  float* flse;           // nullptr or [batch, Hq] fp32
+  const void* extra_out; // [num_extra, batch, Hq, D] out_dtype
+  const float* extra_lse;
+  int64_t sfo_b, sfo_h;
+  int32_t out_dtype, num_extra, lse_column;
 };
 
 struct CombineArgs {
@@ -53,6 +64,7 @@ struct CombineArgs {
   const float* extra_lse;
   int64_t s_mb, s_mh, s_ms, s_ob, s_oh;
   int32_t batch, Hq, D, num_partials, num_extra, mode, mid_dtype, out_dtype;
+  int32_t vec_mid;  // 1: every mid_o row start is 16-byte aligned (128-bit loads allowed)
 };
 
 // ---------------------------------------------------------------- scalar conversions
@@ -75,6 +87,22 @@ __device__ __forceinline__ void store_from_f32(void* p, int64_t idx, int dtype, 
   }
 }
 
+// Agent-scope coherent accesses.  Each XCD has its own L2, and an ordinary store may sit there
+// unseen by the other XCDs until the kernel ends; a relaxed agent-scope atomic store is written
+// through, a relaxed agent-scope atomic load bypasses the local L2.  Workgroups on different
+// XCDs exchange partial results through these instead of cache-wide release/acquire fences,
+// which write back and invalidate a whole L2 each time.
+__device__ __forceinline__ void store_f32_agent(float* p, float x) {
+  __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_f32_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x2 load_f32x2_agent(const float* p) {  // p 8-byte aligned
+  const uint64_t v = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __builtin_bit_cast(f32x2, v);
+}
+
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fd_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -93,30 +121,32 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Decodes blockIdx.x into (sequence, split, kv head, head block) and the split's
-// token range.  Work items are ordered sequence-rank major, then split, then KV
-// head, so workgroups that are dispatched together read neighbouring 16-byte
-// chunks of the same pages.
+// Work item of a workgroup: grid = (Hkv * nhb, S, batch).  blockIdx.x (fastest in dispatch order)
+// walks the KV heads, so workgroups that are dispatched together read neighbouring 256-byte
+// pieces of the same pages; blockIdx.z is the rank of the sequence in the issue order.
 struct WorkItem {
   int b, s, kvh, hb, start, end;
 };
 
 __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   WorkItem w;
-  int bid = blockIdx.x;
-  w.hb = bid % a.nhb;
-  bid /= a.nhb;
-  w.kvh = bid % a.Hkv;
-  bid /= a.Hkv;
-  w.s = bid % a.S;
-  int r = bid / a.S;
+  if (a.nhb == 1) {
+    w.kvh = blockIdx.x;
+    w.hb = 0;
+  } else {
+    w.kvh = blockIdx.x / a.nhb;
+    w.hb = blockIdx.x - w.kvh * a.nhb;
+  }
+  w.s = blockIdx.y;
+  const int r = blockIdx.z;
   int b = a.order ? a.order[r] : r;
   w.b = min(max(b, 0), a.batch - 1);
   int64_t cap = (int64_t)a.max_pages * a.P;
   int64_t len = a.kv_lens[w.b];
   len = len < 0 ? 0 : (len > cap ? cap : len);
-  int kv_len = (int)len;
-  int per = (kv_len + a.S - 1) / a.S;  // ceil(kv_len / S)
+  const int kv_len = (int)len;
+  // per = ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)
+  const int per = (int)(((uint64_t)(uint32_t)(kv_len + a.S - 1) * a.s_magic) >> a.s_shift);
   int64_t st = (int64_t)per * w.s;
   w.start = st > kv_len ? kv_len : (int)st;
   int64_t en = st + per;
@@ -124,10 +154,16 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   return w;
 }
 
+// n / P without a divide or a branch: P is only known at run time, and a branch in the
+// streaming loop would make the compiler's wait counts conservative.
+__device__ __forceinline__ int page_index(const SplitArgs& a, int n) {
+  return (int)(((uint64_t)(uint32_t)n * a.div_magic) >> a.div_shift);
+}
+
 // Flat cache row of logical token n of sequence b: page*P + n%P, with the page id
 // clamped into the pool so that a corrupt table entry cannot fault the GPU.
 __device__ __forceinline__ int token_row(const SplitArgs& a, const int32_t* bt_row, int n) {
-  int pidx = a.log2P >= 0 ? (n >> a.log2P) : (n / a.P);
+  int pidx = page_index(a, n);
   int page = bt_row[pidx];
   page = min(max(page, 0), a.num_pages - 1);
   return page * a.P + (n - pidx * a.P);
@@ -166,18 +202,119 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
     o *= inv;
     const int head = head0 + h;
     const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;
-    if (a.mid_dtype == FD_F32 && a.vec_out) {
-      *(f32x4*)((float*)a.out + off) = o;
+    const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+    if (a.tickets) {
+      // fused combine (fp32 partials only): another XCD's workgroup may read these
+#pragma unroll
+      for (int i = 0; i < 4; ++i) store_f32_agent((float*)a.out + off + i, o[i]);
+      if (d == 0) store_f32_agent(a.lse ? a.lse + ((int64_t)w.b * a.Hq + head) * a.S + w.s : (float*)a.out + off + D, lse);
     } else {
-      for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
-    }
-    if (d == 0) {
-      float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
-      if (a.lse) {
-        a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
+      if (a.mid_dtype == FD_F32 && a.vec_out) {
+        *(f32x4*)((float*)a.out + off) = o;
       } else {
-        store_from_f32(a.out, off + D, a.mid_dtype, lse);
+        for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
       }
+      if (d == 0) {
+        if (a.lse) {
+          a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
+        } else {
+          store_from_f32(a.out, off + D, a.mid_dtype, lse);
+        }
+      }
+    }
+  }
+}
+
+// Fused combine: called by every thread of the workgroup after cta_merge_store() (which, in this
+// mode, wrote the fp32 partials with agent-scope stores).  Every thread waits for its stores to
+// complete, one thread takes a ticket for the (sequence, KV head, head block) group, and the
+// workgroup that draws the last ticket merges the group's S partials (and the extra ones) into the
+// final output with the stand-alone combine kernel's weights softmax(LSE)_s.  No workgroup ever
+// waits for another one.  s_lse: LDS scratch of at least (S + num_extra) * nheads floats.
+template <int D>
+__device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem& w, int head0, int nheads,
+                                              float* s_lse) {
+  __shared__ int s_last;
+  const int tid = threadIdx.x;
+  const int nth = blockDim.x;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // vmcnt(0): the write-through stores have completed
+  __syncthreads();
+  if (tid == 0) {
+    int32_t* t = a.tickets + ((int64_t)w.b * a.Hkv + w.kvh) * a.nhb + w.hb;
+    const int old = __hip_atomic_fetch_add(t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = old == a.S - 1;
+    // every split of the group has arrived: leave the counter clean for the next launch
+    if (last) __hip_atomic_store(t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = last;
+  }
+  __syncthreads();
+  if (!s_last) return;
+
+  const int S = a.S;
+  const int NP = S + a.num_extra;
+  const float* mid = (const float*)a.out;
+  for (int i = tid; i < NP * nheads; i += nth) {
+    const int h = i / NP;
+    const int s = i - h * NP;
+    const int head = head0 + h;
+    float L;
+    if (s < S) {
+      L = load_f32_agent(a.lse ? a.lse + ((int64_t)w.b * a.Hq + head) * S + s
+                               : mid + (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + D);
+    } else {
+      L = a.extra_lse[((int64_t)(s - S) * a.batch + w.b) * a.Hq + head];
+    }
+    s_lse[i] = L;
+  }
+  __syncthreads();
+  constexpr int D4 = D / 4;
+  for (int e = tid; e < nheads * D4; e += nth) {
+    const int h = e / D4;
+    const int d = (e - h * D4) * 4;
+    const int head = head0 + h;
+    const float* ls = s_lse + h * NP;
+    float M = -INFINITY;
+    for (int s = 0; s < NP; ++s) M = fmaxf(M, ls[s]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
+    if (M > -INFINITY) {
+      const float* base = mid + (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + d;
+      // every split slot was written by its workgroup (empty ones hold zeros), so the rows are
+      // loaded unconditionally and several loads stay in flight
+      if (a.vec_out) {
+#pragma unroll 8
+        for (int s = 0; s < S; ++s) {
+          const float wgt = __expf(ls[s] - M);
+          const f32x2 lo = load_f32x2_agent(base + (int64_t)s * a.so_s);
+          const f32x2 hi = load_f32x2_agent(base + (int64_t)s * a.so_s + 2);
+          acc += f32x4{lo[0], lo[1], hi[0], hi[1]} * wgt;
+          L += wgt;
+        }
+      } else {
+#pragma unroll 4
+        for (int s = 0; s < S; ++s) {
+          const float wgt = __expf(ls[s] - M);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) acc[k] += wgt * load_f32_agent(base + (int64_t)s * a.so_s + k);
+          L += wgt;
+        }
+      }
+      for (int x = 0; x < a.num_extra; ++x) {
+        const float wgt = __expf(ls[S + x] - M);
+        const int64_t off = (((int64_t)x * a.batch + w.b) * a.Hq + head) * D + d;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[k] += wgt * load_as_f32(a.extra_out, off + k, a.out_dtype);
+        L += wgt;
+      }
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    const int64_t ob = (int64_t)w.b * a.sfo_b + (int64_t)head * a.sfo_h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) store_from_f32(a.fout, ob + d + k, a.out_dtype, acc[k] * inv);
+    if (d == 0) {
+      const float lse = L > 0.f ? M + __logf(L) : -INFINITY;
+      if (a.lse_column) store_from_f32(a.fout, ob + D, a.out_dtype, lse);
+      if (a.flse) a.flse[(int64_t)w.b * a.Hq + head] = lse;
     }
   }
 }

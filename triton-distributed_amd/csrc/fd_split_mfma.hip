@@ -27,6 +27,8 @@
 //     with v_perm_b32 into the A operand of O^T[dim][head] += V^T . P^T, so the
 //     accumulator also lives in the "lane c = head c" layout and is rescaled
 //     without any cross-lane traffic.
+#include <type_traits>
+
 #include "fd_common.h"
 
 namespace {
@@ -63,8 +65,12 @@ struct Mma<_Float16> {
   }
 };
 
+#ifndef FD_MFMA_OCC
+#define FD_MFMA_OCC
+#endif
+
 template <typename T, bool SOFTCAP>
-__global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a) {
+__global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const SplitArgs a) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -105,17 +111,23 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a)
   float scale2 = a.sm_scale * FD_LOG2E;  // scores are kept in the base-2 domain
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
-  // Row vector of tile t: lane (l & 31) holds the flat cache row of token start + 32t + (l & 31),
-  // tokens past the split end are clamped to the last valid token (their scores are masked).
-  auto tile_rows = [&](int t) -> int {
+  // Block-table entry and in-page slot of tile t for this lane: lane (l & 31) owns token
+  // start + 32t + (l & 31); tokens past the split end are clamped to the last valid token (their
+  // scores are masked).  The table entry is returned raw: its arithmetic is done by the consumer
+  // one iteration later, so the load stays in flight across the tile that is being processed.
+  auto tile_slot = [&](int t, int& slot) -> int {
     int n = w.start + t * kTile + (lane & 31);
     n = min(n, w.end - 1);
-    return token_row(a, bt_row, n);
+    const int pidx = page_index(a, n);
+    slot = n - pidx * a.P;
+    return bt_row[pidx];
   };
 
   u32x4 kraw[8], vraw[8];
   int rows[8];
-  auto fetch_rows = [&](int rv) {
+  auto fetch_rows = [&](int page, int slot) {
+    // flat cache row = page * P + slot, page clamped into the pool so a corrupt table cannot fault
+    const int rv = min(max(page, 0), a.num_pages - 1) * a.P + slot;
 #pragma unroll
     for (int i = 0; i < 8; ++i) rows[i] = __shfl(rv, 4 * g + (i & 3) + 16 * (i >> 2));
   };
@@ -134,16 +146,13 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a)
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  int rv_next = 0;
-  if (t0 < t1) {
-    fetch_rows(tile_rows(t0));
-    issue_k();
-    issue_v();
-    if (t0 + 1 < t1) rv_next = tile_rows(t0 + 1);
-  }
+  int pg_next = 0, slot_next = 0;
 
-  for (int t = t0; t < t1; ++t) {
-    const bool has_next = t + 1 < t1;
+  // One tile.  HAS_NEXT is a compile-time flag (the last tile of the wave is peeled off the loop),
+  // so the steady-state loop has no branch around a load and the wait counts stay exact:
+  // K(t+1) and V(t+1) are in flight while tile t is being computed.
+  auto tile = [&](int t, auto has_next_tag) {
+    constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
     // ---- K tile -> LDS, then start fetching the next tile's K into the freed registers
     wave_lds_fence();
 #pragma unroll
@@ -152,10 +161,14 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a)
       *(u32x4*)(kb + tau * kKRow + c * 16) = kraw[i];
     }
     wave_lds_fence();
-    if (has_next) {
-      fetch_rows(rv_next);
+    if constexpr (HAS_NEXT) {
+      // the machine scheduler must not sink these loads (or hoist later ones) across this point:
+      // the whole pipeline depends on K(t+1) being requested before tile t is computed
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_rows(pg_next, slot_next);
       issue_k();
-      if (t + 2 < t1) rv_next = tile_rows(t + 2);
+      pg_next = tile_slot(min(t + 2, t1 - 1), slot_next);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // ---- S^T = K . Q^T
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -216,10 +229,29 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a)
       for (int e = 0; e < 4; ++e)
         vop[j][e] = __builtin_amdgcn_perm(vraw[2 * e + 1][j >> 1], vraw[2 * e][j >> 1], sel);
     }
-    if (has_next) issue_v();
+    if constexpr (HAS_NEXT) {
+      __builtin_amdgcn_sched_barrier(0);
+      issue_v();
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // ---- O^T += V^T . P^T
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = Mma<T>::run(vop[j], pop, acc[j]);
+  };
+
+  if (t0 < t1) {
+    int slot0;
+    const int pg0 = tile_slot(t0, slot0);
+    pg_next = tile_slot(min(t0 + 1, t1 - 1), slot_next);
+    // same request order as in the loop (table entry of the next tile before the K/V rows), so the
+    // wait counts at the loop head are exact on the first iteration as well
+    __builtin_amdgcn_sched_barrier(0);
+    fetch_rows(pg0, slot0);
+    issue_k();
+    issue_v();
+    __builtin_amdgcn_sched_barrier(0);
+    for (int t = t0; t < t1 - 1; ++t) tile(t, std::true_type{});
+    tile(t1 - 1, std::false_type{});
   }
 
   // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
@@ -241,14 +273,19 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_kernel(const SplitArgs a)
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
   cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, W, w, w.kvh * a.G + w.hb * kHB, nheads, 1.0f);
+  if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);
 }
 
 }  // namespace
 
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
-  const unsigned grid = (unsigned)a.batch * a.S * a.Hkv * a.nhb;
+  const dim3 grid((unsigned)(a.Hkv * a.nhb), (unsigned)a.S, (unsigned)a.batch);
   const unsigned block = 64u * waves;
-  const size_t lds = (size_t)waves * kWaveLds;
+  size_t lds = (size_t)waves * kWaveLds;
+  if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
+    const size_t need = (size_t)(a.S + a.num_extra) * kHB * 4;
+    if (need > lds) lds = need;
+  }
   void (*kern)(const SplitArgs) = nullptr;
   if (kv_dtype == FD_BF16) {
     kern = soft_cap ? fd_split_mfma16_kernel<__bf16, true> : fd_split_mfma16_kernel<__bf16, false>;
@@ -262,6 +299,6 @@ int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, i
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return FD_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(block), lds, stream, a);
+  hipLaunchKernelGGL(kern, grid, dim3(block), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }

@@ -43,7 +43,8 @@ struct KvTraits<FD_F16> {
   static __device__ __forceinline__ void cvt(const u32x4& r, float* f) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      f16x2 h = __builtin_bit_cast(f16x2, r[i]);
+      const uint32_t w = r[i];  // bit_cast of a vector-element lvalue would read element 0
+      f16x2 h = __builtin_bit_cast(f16x2, w);
       f[2 * i] = (float)h[0];
       f[2 * i + 1] = (float)h[1];
     }
@@ -244,11 +245,12 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   }
   __syncthreads();
   cta_merge_store<GH, D>(a, (const float*)smem, PART, W, w, head0, nheads, v_scale);
+  if (a.tickets) fused_combine<D>(a, w, head0, nheads, (float*)smem);
 }
 
 template <int KV, int D>
 int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
-  const unsigned grid = (unsigned)a.batch * a.S * a.Hkv * a.nhb;
+  const dim3 grid((unsigned)(a.Hkv * a.nhb), (unsigned)a.S, (unsigned)a.batch);
   const unsigned block = 64u * waves;
   void (*kern)(const SplitArgs) = nullptr;
   int gh = a.hbsz;
@@ -256,8 +258,12 @@ int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
   else if (gh == 2) kern = fd_split_valu_kernel<KV, D, 2>;
   else if (gh == 4) kern = fd_split_valu_kernel<KV, D, 4>;
   else return FD_ERR_UNSUPPORTED;
-  const size_t lds = (size_t)waves * ((gh * D + 2 * gh + 3) & ~3) * 4;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(block), lds, stream, a);
+  size_t lds = (size_t)waves * ((gh * D + 2 * gh + 3) & ~3) * 4;
+  if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
+    const size_t need = (size_t)(a.S + a.num_extra) * gh * 4;
+    if (need > lds) lds = need;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(block), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }
 

@@ -17,6 +17,9 @@ Keyword-only additions that the reference does not have (all default off):
                   would contribute
   seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
+  fuse_combine    True: one launch, the combine runs in the tail of the split kernel (pays off when
+                  the groups of a ragged batch finish at different times); False (default): split
+                  kernel and combine kernel as two launches
 
 Differences from the reference, on purpose: when ``output_split`` is not
 supplied the partials are kept in fp32 with the LSE in its own fp32 buffer (the
@@ -103,7 +106,7 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
 
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
-            stream=None, path="auto", waves_per_block=0):
+            stream=None, path="auto", waves_per_block=0, fuse_combine=False):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -145,14 +148,6 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
 
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, fd_dtype_of(output_split),
                      fd_dtype_of(output_combine), k_scale, v_scale, path, waves_per_block)
-    check(lib.fd_split_kv(
-        hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_split.data_ptr(),
-        lse_split.data_ptr() if lse_split is not None else None, float(scale), block_table.data_ptr(),
-        kv_lens.data_ptr(), batch,
-        q.stride(0), q.stride(1), k_cache.stride(-3), k_cache.stride(-2), v_cache.stride(-3), v_cache.stride(-2),
-        output_split.stride(0), output_split.stride(1), output_split.stride(2), block_table.stride(0),
-        seq_order.data_ptr() if seq_order is not None else None, byref(p)))
-
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:
@@ -164,15 +159,34 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert ex_lse.is_contiguous() and ex_out.dtype == output_combine.dtype
     if lse_out is not None:
         assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
-    check(lib.fd_combine(
-        hstream, output_split.data_ptr(), lse_split.data_ptr() if lse_split is not None else None,
-        output_combine.data_ptr(), lse_out.data_ptr() if lse_out is not None else None, kv_lens.data_ptr(),
-        batch, q_heads, num_splits,
-        output_split.stride(0), output_split.stride(1), output_split.stride(2),
+    tickets = _tickets(q.device, hstream, batch * q_heads) if fuse_combine else None
+    check(lib.fd_decode(
+        hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_split.data_ptr(),
+        lse_split.data_ptr() if lse_split is not None else None, output_combine.data_ptr(),
+        lse_out.data_ptr() if lse_out is not None else None, float(scale), block_table.data_ptr(),
+        kv_lens.data_ptr(), batch,
+        q.stride(0), q.stride(1), k_cache.stride(-3), k_cache.stride(-2), v_cache.stride(-3), v_cache.stride(-2),
+        output_split.stride(0), output_split.stride(1), output_split.stride(2), block_table.stride(0),
         output_combine.stride(0), output_combine.stride(1),
+        seq_order.data_ptr() if seq_order is not None else None,
         FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
-        ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra, byref(p)))
+        ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra,
+        tickets.data_ptr() if tickets is not None else None, byref(p)))
     return output_combine
+
+
+# Zero-initialised ticket counters of the fused combine, one buffer per (device, stream): calls on
+# different streams may overlap and must not share counters; the kernels leave them at zero.
+_TICKETS = {}
+
+
+def _tickets(device, hstream, n):
+    key = (device.index, hstream)
+    t = _TICKETS.get(key)
+    if t is None or t.numel() < n:
+        t = torch.zeros(max(n, 4096), dtype=torch.int32, device=device)
+        _TICKETS[key] = t
+    return t
 
 
 def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
