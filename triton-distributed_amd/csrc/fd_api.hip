@@ -138,15 +138,17 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   a.vec_out = (p->mid_dtype == FD_F32 && aligned16(out_split) && stride_o_bs % 4 == 0 && stride_o_h % 4 == 0 &&
                stride_o_split % 4 == 0) ? 1 : 0;
 
-  const bool mfma_ok = D == 128 && G >= 4 && (G <= 16 || G % 16 == 0) &&
-                       (p->kv_dtype == FD_BF16 || p->kv_dtype == FD_F16) && p->q_dtype == p->kv_dtype &&
+  const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
+  const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
+  const bool mfma_ok = D == 128 && G >= 4 && (G <= 16 || G % 16 == 0) && q16 &&
+                       (kv_fp8 || p->q_dtype == p->kv_dtype) &&
                        aligned16(q) && stride_q_bs % 8 == 0 && stride_q_h % 8 == 0;
   bool use_mfma = mfma_ok;
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs head_dim 128, group >= 4 (<= 16 or a multiple of 16), 16-bit KV of the "
-                "query's dtype and 16-byte aligned q rows", fn);
+                "%s: MFMA path needs head_dim 128, group >= 4 (<= 16 or a multiple of 16), a 16-bit query with a "
+                "KV cache of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
@@ -155,7 +157,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (use_mfma) {
     a.hbsz = G < 16 ? G : 16;
     a.nhb = (G + 15) / 16;
-    tile = 32;
+    tile = kv_fp8 ? 64 : 32;
   } else {
     a.hbsz = G >= 3 ? 4 : G;
     a.nhb = (G + a.hbsz - 1) / a.hbsz;
@@ -178,8 +180,14 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     }
   }
 
-  int rc = use_mfma ? fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f)
-                    : fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, waves);
+  int rc;
+  if (use_mfma && kv_fp8) {
+    rc = fd_launch_split_mfma_fp8((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
+  } else if (use_mfma) {
+    rc = fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);
+  } else {
+    rc = fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, waves);
+  }
   if (rc == FD_ERR_LAUNCH) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
   if (rc != FD_OK) return fail(rc, "%s: no kernel for kv_dtype %d, head_dim %d, group %d", fn, p->kv_dtype, D, G);
   return FD_OK;

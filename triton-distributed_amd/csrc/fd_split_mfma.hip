@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "fd_common.h"
+#include "fd_mma.h"
 
 namespace {
 
@@ -39,31 +40,6 @@ constexpr int kKRow = 272;        // LDS pitch of a staged K row in bytes (256 +
 constexpr int kWaveLds = kTile * kKRow;  // 8704 B per wave, reused for the wave's partial result
 constexpr int kHB = 16;           // head slots per workgroup (MFMA N)
 static_assert(kWaveLds >= (kHB * kD + 2 * kHB) * 4, "partial result must fit in the K staging buffer");
-
-template <typename T>
-struct Mma;
-template <>
-struct Mma<__bf16> {
-  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
-                                                   0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    f32x2 v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-  }
-};
-template <>
-struct Mma<_Float16> {
-  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
-                                                  0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    f32x2 v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
-  }
-};
 
 #ifndef FD_MFMA_OCC
 #define FD_MFMA_OCC

@@ -1,0 +1,281 @@
+// Split-KV GQA paged decode on MFMA with an fp8-e4m3 (OCP) KV cache (gfx950), head_dim 128.
+//
+// New functionality relative to the reference, whose split kernel
+// (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) would cast an fp8
+// cache with `k.to(q.dtype)` and no scales (:208) and round P to fp8 (:230).
+// Here K and V bytes are dequantised in registers -- v_cvt_scalef32_pk_{bf16,f16}_fp8
+// turns two e4m3 bytes into two packed 16-bit values exactly -- and fed to the same
+// 16x16x32 MFMA as the 16-bit kernel; the per-KV-head K scale is folded into the
+// softmax scale and the V scale is applied once to the finished partial.
+//
+// Geometry per wave (lane = 16*g + m): 64-token tiles (8 KB of K and 8 KB of V).
+//   * K: 8 x global_load_dwordx4, eight whole 128-byte rows per instruction; staged
+//     in LDS (row pitch 144 B) and read back as the MFMA A operand with ds_read_b64
+//     (lane (g, m) <- token m's bytes 32*ks + 8g .. +7), converted, multiplied with Q.
+//   * Scores S^T[token][head]: four 16-token sub-tiles; lane (g, c) ends up with head
+//     c's scores for tokens 16*tt + 4g + i.
+//   * V: 16 x global_load_dwordx2.  For P.V the 64 tokens form two K=32 MFMA blocks;
+//     block kb takes tokens tau(g,e,kb) = 16*(2kb + e/4) + 4g + e%4, which are exactly
+//     the tokens whose probabilities lane (g, .) holds.  Lane (g, m = 8u + cc) loads the
+//     8 bytes 16*cc + 8u .. +7 of those rows (the two u-halves of a wave row read one
+//     contiguous 16 bytes, the eight cc a whole row), converts them and transposes the
+//     8x8 block with v_perm_b32 into 8 A operands of O^T[dim][head] += V^T . P^T.
+#include <type_traits>
+
+#include "fd_common.h"
+#include "fd_mma.h"
+
+namespace {
+
+constexpr int kD = 128;
+constexpr int kTile = 64;         // tokens per tile
+constexpr int kKRow = 144;        // LDS pitch of a staged fp8 K row in bytes (128 + 16 pad)
+constexpr int kWaveLds = kTile * kKRow;  // 9216 B per wave, reused for the wave's partial result
+constexpr int kHB = 16;
+static_assert(kWaveLds >= (kHB * kD + 2 * kHB) * 4, "partial result must fit in the K staging buffer");
+
+template <typename T, bool SOFTCAP>
+__global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs a) {
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int W = blockDim.x >> 6;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const WorkItem w = decode_work_item(a);
+  const int ntok = w.end - w.start;
+  const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
+  const int tpw = (ntiles + W - 1) / W;
+  const int t0 = wave * tpw;
+  const int t1 = min(t0 + tpw, ntiles);
+
+  const int head_in_group = w.hb * kHB + c;
+  const bool head_ok = head_in_group < a.G;
+  const int head = w.kvh * a.G + head_in_group;
+
+  u32x4 qop[4];  // Q as the MFMA B operand: lane (g, c) holds Q[head c][32*ks + 8g .. +7]
+  {
+    const char* qp = (const char*)a.q + ((int64_t)w.b * a.sq_b + (int64_t)head * a.sq_h) * 2;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qop[ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
+    }
+  }
+
+  const int32_t* bt_row = a.bt + (int64_t)w.b * a.sbt;
+  // K: lane reads the 16-byte chunk (lane & 7) of token 8i + (lane >> 3); V: 8 bytes at 16*cc + 8u
+  const char* kbase = (const char*)a.k + (int64_t)w.kvh * a.sk_h + (lane & 7) * 16;
+  const char* vbase = (const char*)a.v + (int64_t)w.kvh * a.sv_h + (c & 7) * 16 + (c >> 3) * 8;
+  const int k_pitch = (int)a.sk_t;
+  const int v_pitch = (int)a.sv_t;
+  char* kb = smem + wave * kWaveLds;
+
+  const float kq_scale = a.sm_scale * a.k_scale[w.kvh];  // K dequantisation folded into the softmax scale
+  const float scale2 = kq_scale * FD_LOG2E;
+  const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
+
+  // lane l owns token start + 64t + l of tile t (clamped to the last valid token of the split)
+  auto tile_slot = [&](int t, int& slot) -> int {
+    int n = w.start + t * kTile + lane;
+    n = min(n, w.end - 1);
+    const int pidx = page_index(a, n);
+    slot = n - pidx * a.P;
+    return bt_row[pidx];
+  };
+  auto flat_row = [&](int page, int slot) -> int {
+    return min(max(page, 0), a.num_pages - 1) * a.P + slot;
+  };
+
+  u32x4 kraw[8];
+  u32x2 vraw[16];
+  auto issue_k = [&](int rv) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = __shfl(rv, 8 * i + (lane >> 3));
+      kraw[i] = *(const u32x4*)(kbase + (int64_t)row * k_pitch);
+    }
+  };
+  auto issue_v = [&](int rv, int kblk) {  // the 8 rows of P.V block kblk
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int row = __shfl(rv, 16 * (2 * kblk + (e >> 2)) + 4 * g + (e & 3));
+      vraw[8 * kblk + e] = *(const u32x2*)(vbase + (int64_t)row * v_pitch);
+    }
+  };
+
+  float m = -INFINITY;
+  float l = 0.f;
+  f32x4 acc[8];  // acc[j][i] = O[head c][dim 16*(r & 7) + 8*(r >> 3) + j], r = 4g + i
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int pg_next = 0, slot_next = 0;
+  int rv_cur = 0;  // flat rows of the tile whose V is still to be requested
+
+  auto tile = [&](int t, auto has_next_tag) {
+    constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+    // ---- K tile -> LDS, then request the next tile's K
+    wave_lds_fence();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *(u32x4*)(kb + (8 * i + (lane >> 3)) * kKRow + (lane & 7) * 16) = kraw[i];
+    wave_lds_fence();
+    if constexpr (HAS_NEXT) {
+      __builtin_amdgcn_sched_barrier(0);
+      rv_cur = flat_row(pg_next, slot_next);
+      issue_k(rv_cur);
+      pg_next = tile_slot(min(t + 2, t1 - 1), slot_next);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- S^T = K . Q^T, four 16-token sub-tiles
+    f32x4 s[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        const u32x2 kk = *(const u32x2*)(kb + (16 * tt + c) * kKRow + (4 * ks + g) * 8);
+        const uint32_t k0 = kk[0], k1 = kk[1];
+        u32x4 ak = {Mma<T>::from_fp8(k0, false), Mma<T>::from_fp8(k0, true), Mma<T>::from_fp8(k1, false),
+                    Mma<T>::from_fp8(k1, true)};
+        s[tt] = Mma<T>::run(ak, qop[ks], s[tt]);
+      }
+    }
+    // ---- online softmax: x[4*tt + i] <-> token 16*tt + 4g + i, head c
+    float x[16];
+    const int n0 = w.start + t * kTile;
+    const bool full = n0 + kTile <= w.end;
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = s[tt][i];
+        if (SOFTCAP) {
+          v = fd_softcap(v * kq_scale, a.soft_cap, inv_cap) * FD_LOG2E;
+        } else {
+          v *= scale2;
+        }
+        x[4 * tt + i] = (full || n0 + 16 * tt + 4 * g + i < w.end) ? v : -INFINITY;
+      }
+    }
+    float mx = x[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, x[i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fd_exp2(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      x[i] = fd_exp2(x[i] - m_new);
+      psum += x[i];
+    }
+    l = l * alpha + psum;
+    if (__any(m_new > m)) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+    }
+    m = m_new;
+    u32x4 pop[2];  // P^T B operands: block kb, element e <-> token 16*(2kb + e/4) + 4g + e%4
+#pragma unroll
+    for (int kblk = 0; kblk < 2; ++kblk)
+#pragma unroll
+      for (int q2 = 0; q2 < 4; ++q2) pop[kblk][q2] = Mma<T>::pack(x[8 * kblk + 2 * q2], x[8 * kblk + 2 * q2 + 1]);
+
+    // ---- V: dequantise, transpose 8 tokens x 8 dims per block, O^T += V^T . P^T
+#pragma unroll
+    for (int kblk = 0; kblk < 2; ++kblk) {
+      uint32_t cv[8][4];  // cv[e][jp] = dims (2jp, 2jp+1) of token e as packed 16-bit
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t v0 = vraw[8 * kblk + e][0], v1 = vraw[8 * kblk + e][1];
+        cv[e][0] = Mma<T>::from_fp8(v0, false);
+        cv[e][1] = Mma<T>::from_fp8(v0, true);
+        cv[e][2] = Mma<T>::from_fp8(v1, false);
+        cv[e][3] = Mma<T>::from_fp8(v1, true);
+      }
+      if constexpr (HAS_NEXT) {
+        // this block's V registers have just been consumed: refill them in place with the next tile's rows
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(rv_cur, kblk);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 vop;
+#pragma unroll
+        for (int q2 = 0; q2 < 4; ++q2) vop[q2] = __builtin_amdgcn_perm(cv[2 * q2 + 1][j >> 1], cv[2 * q2][j >> 1], sel);
+        acc[j] = Mma<T>::run(vop, pop[kblk], acc[j]);
+      }
+    }
+  };
+
+  if (t0 < t1) {
+    int slot0;
+    const int pg0 = tile_slot(t0, slot0);
+    pg_next = tile_slot(min(t0 + 1, t1 - 1), slot_next);
+    __builtin_amdgcn_sched_barrier(0);
+    rv_cur = flat_row(pg0, slot0);
+    issue_k(rv_cur);
+    issue_v(rv_cur, 0);
+    issue_v(rv_cur, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int t = t0; t < t1 - 1; ++t) tile(t, std::true_type{});
+    tile(t1 - 1, std::false_type{});
+  }
+
+  // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  wave_lds_fence();
+  float* part = (float*)kb;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * g + i;
+    const int dim0 = 16 * (r & 7) + 8 * (r >> 3);
+    f32x4 lo = {acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
+    f32x4 hi = {acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
+    *(f32x4*)(part + c * kD + dim0) = lo;
+    *(f32x4*)(part + c * kD + dim0 + 4) = hi;
+  }
+  if (g == 0) {
+    part[kHB * kD + c] = m;
+    part[kHB * kD + kHB + c] = l;
+  }
+  __syncthreads();
+  const int nheads = min(kHB, a.G - w.hb * kHB);
+  const int head0 = w.kvh * a.G + w.hb * kHB;
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, W, w, head0, nheads, a.v_scale[w.kvh]);
+  if (a.tickets) fused_combine<kD>(a, w, head0, nheads, (float*)smem);
+}
+
+}  // namespace
+
+int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap) {
+  const dim3 grid((unsigned)(a.Hkv * a.nhb), (unsigned)a.S, (unsigned)a.batch);
+  const unsigned block = 64u * waves;
+  size_t lds = (size_t)waves * kWaveLds;
+  if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
+    const size_t need = (size_t)(a.S + a.num_extra) * kHB * 4;
+    if (need > lds) lds = need;
+  }
+  void (*kern)(const SplitArgs) = nullptr;
+  if (q_dtype == FD_BF16) {
+    kern = soft_cap ? fd_split_mfma_fp8_kernel<__bf16, true> : fd_split_mfma_fp8_kernel<__bf16, false>;
+  } else if (q_dtype == FD_F16) {
+    kern = soft_cap ? fd_split_mfma_fp8_kernel<_Float16, true> : fd_split_mfma_fp8_kernel<_Float16, false>;
+  } else {
+    return FD_ERR_UNSUPPORTED;
+  }
+  if (lds > 64 * 1024) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return FD_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(block), lds, stream, a);
+  return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
+}
