@@ -40,6 +40,12 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
+    ap.add_argument("--copy-ref", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times: a kernel of known traffic against which "
+                         "a counter run (FETCH_SIZE / WRITE_SIZE) of this same command is scaled")
+    ap.add_argument("--traffic-json", default=None,
+                    help="JSON file {\"traffic\": bytes per split-kernel launch} measured with the counter runs; "
+                         "copied into roofline.traffic")
     return ap.parse_args()
 
 
@@ -145,6 +151,27 @@ def main():
     split_us = e0.elapsed_time(e1) * 1e3 / args.steps
     achieved = algo_bytes / (split_us * 1e-6) / 1e9
 
+    if args.copy_ref:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    # HBM bytes per split-kernel launch from the committed counter runs (profiles/*__hbm_traffic.json,
+    # FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None when this workload has none
+    traffic = None
+    import glob
+    candidates = [args.traffic_json] if args.traffic_json else sorted(
+        glob.glob(os.path.join(ROOT, "profiles", "*__hbm_traffic.json")))
+    for path in candidates:
+        if path and os.path.exists(path):
+            with open(path) as f:
+                rec = json.load(f)
+            if args.traffic_json or (rec.get("workload") == wl.name and args.path == "auto"):
+                traffic = rec.get("traffic")
+                break
+
     # ---- result of pool 0 for the check against the CPU baseline
     step(0)
     torch.cuda.synchronize()
@@ -174,7 +201,7 @@ def main():
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
         "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel_us": round(split_us, 3)},
+                     "traffic": traffic, "kernel_us": round(split_us, 3)},
     }
 
     if not args.no_cpu_baseline:

@@ -1,0 +1,165 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every symbol declared in
+include/flash_decode.h, argument validation returns error codes (no compute call is made without
+a GPU), the ctypes mirror of fd_params matches the header, and the host-side helpers behave."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flash_decode.h")
+
+
+def _header_text():
+    with open(HEADER) as f:
+        return f.read()
+
+
+def test_library_exports_every_declared_symbol(fd):
+    lib = fd.load_library()
+    declared = re.findall(r"FD_API\s+[\w\s\*]+?\b(fd_\w+)\s*\(", _header_text())
+    assert set(declared) == set(fd._lib.EXPORTED_SYMBOLS), declared
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.fd_abi_version() == int(re.search(r"#define FD_ABI_VERSION (\d+)", _header_text()).group(1))
+
+
+def test_enums_and_params_struct_mirror_the_header(fd):
+    text = _header_text()
+    L = fd._lib
+    enums = dict(re.findall(r"\b(FD_[A-Z0-9_]+)\s*=\s*(-?\d+)", text))
+    for name in ("FD_F32", "FD_F16", "FD_BF16", "FD_FP8_E4M3", "FD_PATH_AUTO", "FD_PATH_VALU", "FD_PATH_MFMA",
+                 "FD_COMBINE_SPLIT", "FD_COMBINE_SPLIT_LSE", "FD_COMBINE_RANK"):
+        assert int(enums[name]) == getattr(L, name), name
+    body = re.search(r"typedef struct fd_params \{(.*?)\} fd_params;", text, re.S).group(1)
+    fields = re.findall(r"^\s*(?:const\s+)?(int32_t|float)\s*(\*?)\s*(\w+);", body, re.M)
+    mirror = [(n, t) for n, t in L.FdParams._fields_]
+    assert [f[2] for f in fields] == [n for n, _ in mirror]
+    for (ctype, ptr, name), (_, pytype) in zip(fields, mirror):
+        expect = ctypes.c_void_p if ptr else (ctypes.c_int32 if ctype == "int32_t" else ctypes.c_float)
+        assert pytype is expect, name
+
+
+def test_invalid_arguments_return_error_codes_without_touching_a_gpu(fd):
+    lib = fd.load_library()
+    L = fd._lib
+    p = L.FdParams()
+    # NULL tensors
+    rc = lib.fd_split_kv(None, None, None, None, None, None, 1.0, None, None, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None,
+                         ctypes.byref(p))
+    assert rc == -1 and b"NULL" in lib.fd_last_error()
+    rc = lib.fd_split_kv(None, None, None, None, None, None, 1.0, None, None, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None, None)
+    assert rc == -1 and b"params" in lib.fd_last_error()
+    fake = ctypes.c_void_p(0x1000)   # never dereferenced: validation fails first
+    p.q_heads, p.kv_heads = 6, 4     # not a multiple
+    rc = lib.fd_split_kv(None, fake, fake, fake, fake, None, 1.0, fake, fake, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None,
+                         ctypes.byref(p))
+    assert rc == -1 and b"multiple" in lib.fd_last_error()
+    p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits, p.num_pages, p.max_pages_per_seq = 8, 2, 96, 16, 4, 8, 4
+    rc = lib.fd_split_kv(None, fake, fake, fake, fake, None, 1.0, fake, fake, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None,
+                         ctypes.byref(p))
+    assert rc == -2 and b"head_dim" in lib.fd_last_error()
+    p.head_dim, p.q_dtype, p.kv_dtype, p.mid_dtype = 128, L.FD_BF16, L.FD_FP8_E4M3, L.FD_F32
+    rc = lib.fd_split_kv(None, fake, fake, fake, fake, None, 1.0, fake, fake, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None,
+                         ctypes.byref(p))
+    assert rc == -1 and b"k_scale" in lib.fd_last_error()
+    p.kv_dtype = L.FD_BF16
+    rc = lib.fd_split_kv(None, fake, ctypes.c_void_p(0x1008), fake, fake, None, 1.0, fake, fake, 1, 1024, 128, 1024,
+                         128, 1024, 128, 0, 0, 0, 4, None, ctypes.byref(p))
+    assert rc == -3 and b"aligned" in lib.fd_last_error()
+    p.num_pages, p.page_size = 1 << 20, 1 << 12
+    rc = lib.fd_split_kv(None, fake, fake, fake, fake, None, 1.0, fake, fake, 1, 1024, 128, 1024, 128, 1024, 128, 0, 0,
+                         0, 4, None, ctypes.byref(p))
+    assert rc == -5
+    # combine / schedule / decode
+    assert lib.fd_combine(None, None, None, None, None, None, 1, 1, 1, 0, 0, 0, 0, 0, 0, None, None, 0,
+                          ctypes.byref(p)) == -1
+    assert lib.fd_combine(None, fake, None, fake, None, fake, 1, 8, 4, 0, 0, 0, 0, 0, 7, None, None, 0,
+                          ctypes.byref(p)) == -1 and b"mode" in lib.fd_last_error()
+    assert lib.fd_schedule(None, None, 4, None) == -1
+    assert lib.fd_decode(None, fake, fake, fake, fake, None, None, None, 1.0, fake, fake, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                         0, 0, 0, None, 0, None, None, 0, None, ctypes.byref(p)) == -1
+    # batch == 0 is a no-op success
+    p2 = L.FdParams()
+    assert lib.fd_schedule(None, fake, 0, fake) == 0
+
+
+def test_wrappers_refuse_cpu_tensors_loudly(fd):
+    wl = fd.utils.make_config(1, scale_down=8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        fd.gqa_fwd_batch_decode(wl.q, wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, wl.scale)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        fd.schedule_sequences(wl.kv_lens)
+    layer = fd.SpGQAFlashDecodeAttention(0, 0, 2, 1, 8, 2, 128, 128, page_size=128, max_allowed_batch=1)
+    with pytest.raises(RuntimeError, match="remote_partials"):
+        layer(wl.q, wl.k_cache, wl.v_cache, torch.ones(2, 1, dtype=torch.int32), wl.block_table)
+
+
+def test_missing_library_is_an_error_not_a_fallback(fd, tmp_path, monkeypatch):
+    monkeypatch.setattr(fd._lib, "_lib", None)
+    with pytest.raises(RuntimeError, match="not built"):
+        fd._lib.load_library(str(tmp_path / "nope.so"))
+    monkeypatch.undo()
+    fd.load_library()
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "triton-distributed_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                with open(os.path.join(dirpath, f)) as fh:
+                    text = fh.read()
+                assert not re.search(r"^\s*(import|from)\s+oracle\b", text, re.M), f
+
+
+def test_reference_names_are_exported(fd):
+    for name in ("gqa_fwd_batch_decode", "gqa_fwd_batch_decode_aot", "gqa_fwd_batch_decode_intra_rank",
+                 "gqa_fwd_batch_decode_intra_rank_aot", "gqa_fwd_batch_decode_persistent",
+                 "gqa_fwd_batch_decode_persistent_aot", "kernel_inter_rank_gqa_fwd_batch_decode_combine_kv",
+                 "get_triton_combine_kv_algo_info"):
+        assert hasattr(fd.kernels, name)
+    assert hasattr(fd.layers, "SpGQAFlashDecodeAttention")
+    import triton_dist_amd
+    from triton_dist_amd.kernels import gqa_fwd_batch_decode  # noqa: F401
+    assert triton_dist_amd is fd
+    info = fd.kernels.get_triton_split_kv_algo_info(32, 8, 128, 128, 16)
+    assert info["kv_group_num"] == 4 and info["NUM_KV_SPLITS"] == 32 and info["path"] == "mfma"
+    assert fd.kernels.get_triton_combine_kv_algo_info(split_kv=16)["NUM_KV_SPLITS"] == 16
+
+
+def test_workload_generators_and_algorithmic_bytes(fd):
+    wl = fd.utils.make_config(2, scale_down=64)
+    assert wl.q.shape == (8, 32, 128) and wl.k_cache.shape[1:] == (16, 8, 128) and wl.kv_split == 32
+    # every page referenced exactly once (a permutation of the pool)
+    used = torch.cat([wl.block_table[b, :8] for b in range(8)])
+    assert sorted(used.tolist()) == list(range(64))
+    # bytes formula: K+V once, Q, used table entries, kv_lens, output, fp32 LSE
+    n = 128
+    expect = 8 * n * 8 * 256 * 2 + 8 * 32 * 128 * 2 + 8 * (n // 16) * 4 + 8 * 4 + 8 * 32 * 128 * 2 + 8 * 32 * 4
+    assert wl.algorithmic_bytes() == expect
+    wl5 = fd.utils.make_config(5, scale_down=64)
+    assert wl5.k_cache.dtype == torch.float8_e4m3fn and wl5.k_scale.shape == (8,)
+    assert wl5.algorithmic_bytes() == (wl5.kv_lens.sum().item() * 8 * 256 + 64 * 128 * 2 * wl5.q.shape[0] +
+                                       sum(-(-int(x) // 16) for x in wl5.kv_lens) * 4 + 4 * wl5.q.shape[0] +
+                                       wl5.q.shape[0] * 64 * 128 * 2 + wl5.q.shape[0] * 64 * 4 + 64)
+    wl3 = fd.utils.make_config(3, scale_down=64)
+    assert wl3.extra_out.shape == (7, 1, 32, 128) and float(wl3.extra_lse.min()) >= 5 and float(wl3.extra_lse.max()) <= 15
+    wl4 = fd.utils.make_config(4, scale_down=16)
+    assert len(set(wl4.kv_lens.tolist())) > 1          # ragged
+
+
+def test_sp_layer_staging_ring_grows_and_shrinks(fd):
+    layer = fd.SpGQAFlashDecodeAttention(1, 0, 4, 1, 8, 2, 128, 128, max_allowed_batch=64,
+                                         thrink_buffer_threshold=3, stages=2)
+    base = layer.max_allgather_buffer_size
+    assert base == 4 * 8 * 128 * 8                        # sp_flash_decode_layer.py:68
+    st = layer._stage(base + 1, torch.device("cpu"))
+    assert layer.max_allgather_buffer_size == 2 * base and st.numel() == base + 1
+    for _ in range(3):
+        layer._stage(16, torch.device("cpu"))
+    assert layer.max_allgather_buffer_size == base
+    layer.finalize()
+    assert layer.ag_buffer is None
