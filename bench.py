@@ -37,6 +37,8 @@ def parse_args():
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
     ap.add_argument("--fuse", action="store_true", help="fuse the combine into the tail of the split kernel")
+    ap.add_argument("--exact-splits", action="store_true",
+                    help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
@@ -94,6 +96,8 @@ def main():
         kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
     if wl.extra_out is not None:
         kw.update(extra_partials=(wl.extra_out, wl.extra_lse))
+    if args.exact_splits:
+        kw["plan_splits"] = False
     fn = fd.gqa_fwd_batch_decode_persistent if args.variant == "persistent" else fd.gqa_fwd_batch_decode
     if args.variant == "persistent":
         kw["seq_order"] = torch.empty(B, dtype=torch.int32, device=dev)
@@ -124,11 +128,13 @@ def main():
     from ctypes import byref
     lib = fd.load_library()
     fk = importlib.import_module("triton-distributed_amd.kernels.flash_decode")
-    n_o = B * Hq * S * D
-    mid = workspace[:n_o].view(B, Hq, S, D)
-    lse_split = workspace[n_o:n_o + B * Hq * S].view(B, Hq, S)
     p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
                         wl.k_scale, wl.v_scale, args.path, args.waves)
+    S_eff = S if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
+    p.num_splits = S_eff
+    n_o = B * Hq * S_eff * D
+    mid = workspace[:n_o].view(B, Hq, S_eff, D)
+    lse_split = workspace[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
     hstream = torch.cuda.current_stream().cuda_stream
     order_ptr = kw["seq_order"].data_ptr() if args.variant == "persistent" else None
 
@@ -192,7 +198,7 @@ def main():
                  f"{str(wl.q.dtype).replace('torch.', '')} KV+Q, fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "q_heads": Hq, "kv_heads": wl.k_cache.shape[2], "head_dim": D,
-                   "page_size": wl.k_cache.shape[1], "kv_splits": S,
+                   "page_size": wl.k_cache.shape[1], "kv_splits": S, "kv_splits_used": S_eff,
                    "kv_len_total": int(wl_cpu.kv_lens.sum()), "kv_pools_rotated": len(pools),
                    "variant": args.variant, "path": args.path, "fused_combine": args.fuse},
         "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),

@@ -196,6 +196,19 @@ FD_API int fd_decode(void* stream, const void* q, const void* k_cache, const voi
  */
 FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* seq_order);
 
+/*
+ * How many splits the library would use for a decode step whose partials the caller does
+ * not look at.  NUM_KV_SPLITS is a tuning constant in the reference (flash_decode.py:779:
+ * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
+ * the partial workspace is internal, fewer and longer splits mean fewer workgroup
+ * prologues and fewer partials for the combine.  Returns min(params->num_splits, the split
+ * count that (1) puts one wave on every wave slot of the chip and (2) keeps every
+ * workgroup at or below 2048 tokens of a full-length sequence), or a negative fd_status.
+ * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
+ * params->num_splits splits with the reference's ranges.
+ */
+FD_API int fd_plan_splits(const fd_params* params, int32_t batch);
+
 /* Message for the last non-zero status returned on this thread ("" if none). */
 FD_API const char* fd_last_error(void);
 

@@ -24,7 +24,8 @@ FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_last_error", "fd_abi_version")
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_plan_splits", "fd_last_error",
+                    "fd_abi_version")
 
 _DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
 if hasattr(torch, "float8_e4m3fn"):
@@ -83,6 +84,8 @@ def load_library(path: str = None) -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
         c_int32, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p,
         c_int32, c_void_p, POINTER(FdParams)]
+    lib.fd_plan_splits.restype = c_int32
+    lib.fd_plan_splits.argtypes = [POINTER(FdParams), c_int32]
     lib.fd_schedule.restype = c_int32
     lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]
     lib.fd_last_error.restype = c_char_p

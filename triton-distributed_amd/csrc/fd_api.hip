@@ -76,6 +76,11 @@ struct FusedTail {          // what the fused combine needs on top of the split 
   int32_t num_extra = 0, lse_column = 0;
 };
 
+// fd_plan_splits: wave slots of one MI355X at the split kernels' occupancy (256 CUs x 4 SIMDs x 2 waves) and the
+// largest token count one workgroup should own (keeps a ragged batch balanceable by the dispatcher).
+constexpr int64_t kResidentWaves = 2048;
+constexpr int64_t kMaxTokensPerGroup = 2048;
+
 // Largest dynamic LDS a workgroup may ask for on gfx950 (160 KB per CU).
 constexpr size_t kMaxLds = 160 * 1024;
 
@@ -166,10 +171,25 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
   const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
-  const int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
+  int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
+  // Adjacent KV heads per workgroup (one wave each): sibling waves then fetch up to 512 contiguous bytes
+  // of every token row together.  Only the MFMA kernels, and not with the fused combine (its tickets
+  // are per KV head).
+  a.hpw = 1;
+  const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
+  if (use_mfma && !fuse) {
+    const int row_bytes = D * kvsz;
+    int h = 512 / row_bytes;
+    const char* env = getenv("FD_HEADS_PER_BLOCK");
+    if (env && atoi(env) > 0) h = atoi(env);
+    while (h > 1 && (a.Hkv % h != 0 || h * waves > 8)) h >>= 1;
+    if (h < 1) h = 1;
+    a.hpw = h;
+  }
+  waves *= a.hpw;   // total waves of a workgroup
 
   // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS
-  if (tail && tail->tickets && p->mid_dtype == FD_F32) {  // the fused tail exchanges fp32 partials only
+  if (fuse) {  // the fused tail exchanges fp32 partials only
     const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (use_mfma ? 16 : a.hbsz) * 4;
     if (lse_lds <= kMaxLds / 2) {
       a.tickets = tail->tickets; a.fout = tail->out; a.flse = tail->lse_out;
@@ -234,6 +254,27 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
   return fd_combine(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
                     stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out, extra_lse,
                     num_extra, p);
+}
+
+int fd_plan_splits(const fd_params* p, int32_t batch) {
+  if (!p) return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: params is NULL");
+  if (batch <= 0 || p->q_heads <= 0 || p->kv_heads <= 0 || p->q_heads % p->kv_heads != 0 || p->num_splits <= 0 ||
+      p->page_size <= 0 || p->max_pages_per_seq <= 0)
+    return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0");
+  const int G = p->q_heads / p->kv_heads;
+  const bool mfma = p->head_dim == 128 && G >= 4 && (G <= 16 || G % 16 == 0) && p->path != FD_PATH_VALU &&
+                    (p->kv_dtype == FD_FP8_E4M3 || p->kv_dtype == FD_F16 || p->kv_dtype == FD_BF16);
+  const int64_t nhb = mfma ? (G + 15) / 16 : (G + (G >= 3 ? 4 : G) - 1) / (G >= 3 ? 4 : G);
+  const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // workgroups per split
+  const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
+  // (1) enough splits to put one wave on every wave slot of the chip (256 CUs x 8 waves) ...
+  int64_t s_fill = (kResidentWaves + groups - 1) / groups;
+  // (2) ... and enough that no workgroup owns more than kMaxTokensPerGroup tokens of a full-length sequence
+  int64_t s_bal = (max_tokens + kMaxTokensPerGroup - 1) / kMaxTokensPerGroup;
+  int64_t s = s_fill > s_bal ? s_fill : s_bal;
+  if (s > p->num_splits) s = p->num_splits;
+  if (s < 1) s = 1;
+  return (int)s;
 }
 
 int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,

@@ -51,15 +51,14 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int W = blockDim.x >> 6;
   const int g = lane >> 4;
   const int c = lane & 15;
 
-  const WorkItem w = decode_work_item(a);
+  const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
-  const int tpw = (ntiles + W - 1) / W;
-  const int t0 = wave * tpw;
+  const int tpw = (ntiles + w.nsub - 1) / w.nsub;
+  const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 
   const int head_in_group = w.hb * kHB + c;
@@ -248,14 +247,14 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, W, w, w.kvh * a.G + w.hb * kHB, nheads, 1.0f);
-  if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads, false);
+  if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
 }
 
 }  // namespace
 
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
-  const dim3 grid((unsigned)(a.Hkv * a.nhb), (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid((unsigned)(a.Hkv / a.hpw * a.nhb), (unsigned)a.S, (unsigned)a.batch);  // waves = hpw heads x sub-ranges
   const unsigned block = 64u * waves;
   size_t lds = (size_t)waves * kWaveLds;
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS

@@ -82,15 +82,14 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int W = blockDim.x >> 6;
   const int rg = lane / LPR;          // lane group = row within a load instruction
   const int c = lane % LPR;           // chunk of the row
 
-  const WorkItem w = decode_work_item(a);
+  const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + TILE - 1) / TILE : 0;
-  const int tpw = (ntiles + W - 1) / W;
-  const int t0 = wave * tpw;
+  const int tpw = (ntiles + w.nsub - 1) / w.nsub;
+  const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 
   const int head0 = w.kvh * a.G + w.hb * GH;
@@ -98,11 +97,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 
   // q[h][c*E .. c*E+E) in fp32, pre-multiplied by the softmax scale (and the K dequant scale).
   float kq_scale = a.sm_scale;
-  float v_scale = 1.0f;
-  if (KV == FD_FP8_E4M3) {
-    kq_scale *= a.k_scale[w.kvh];
-    v_scale = a.v_scale[w.kvh];
-  }
+  if (KV == FD_FP8_E4M3) kq_scale *= a.k_scale[w.kvh];   // the V scale multiplies the finished partial
   const bool softcap = a.soft_cap > 0.f;
   const float inv_cap = softcap ? 1.0f / a.soft_cap : 0.f;
   const float post = softcap ? 1.0f : FD_LOG2E;  // without soft-cap scores go straight to base 2
@@ -244,13 +239,13 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
     }
   }
   __syncthreads();
-  cta_merge_store<GH, D>(a, (const float*)smem, PART, W, w, head0, nheads, v_scale);
-  if (a.tickets) fused_combine<D>(a, w, head0, nheads, (float*)smem);
+  cta_merge_store<GH, D>(a, (const float*)smem, PART, w, nheads, KV == FD_FP8_E4M3);
+  if (a.tickets) fused_combine<D>(a, w, head0, nheads, (float*)smem);  // hpw == 1 when fused
 }
 
 template <int KV, int D>
 int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
-  const dim3 grid((unsigned)(a.Hkv * a.nhb), (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid((unsigned)(a.Hkv / a.hpw * a.nhb), (unsigned)a.S, (unsigned)a.batch);  // waves = hpw heads x sub-ranges
   const unsigned block = 64u * waves;
   void (*kern)(const SplitArgs) = nullptr;
   int gh = a.hbsz;

@@ -17,6 +17,10 @@ Keyword-only additions that the reference does not have (all default off):
                   would contribute
   seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
+  plan_splits     True (default): when ``output_split`` is not supplied, ``kv_split`` is an upper bound
+                  and the library uses ``fd_plan_splits`` splits (same result, fewer workgroup prologues
+                  and partials); False: exactly ``kv_split`` splits.  With a caller-supplied
+                  ``output_split`` the split count and ranges are always the reference's.
   fuse_combine    True: one launch, the combine runs in the tail of the split kernel (pays off when
                   the groups of a ragged batch finish at different times); False (default): split
                   kernel and combine kernel as two launches
@@ -34,7 +38,7 @@ from typing import Optional
 
 import torch
 
-from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
+from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F32, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
                     FdParams, check, fd_dtype_of, load_library, stream_handle)
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
@@ -106,7 +110,7 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
 
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
-            stream=None, path="auto", waves_per_block=0, fuse_combine=False):
+            stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -126,6 +130,13 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
 
     lse_split = None
     if output_split is None:
+        if plan_splits:
+            # nobody looks at the partials: let the library merge splits (fewer, longer ones)
+            plan = _make_params(q, k_cache, block_table, num_splits, soft_cap, FD_F32, FD_F32, k_scale, v_scale, path,
+                                waves_per_block)
+            num_splits = lib.fd_plan_splits(byref(plan), batch)
+            if num_splits < 0:
+                check(num_splits)
         # internal partials: fp32, 128-bit aligned rows, LSE in its own buffer
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
