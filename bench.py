@@ -37,6 +37,7 @@ def parse_args():
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
     ap.add_argument("--fuse", action="store_true", help="fuse the combine into the tail of the split kernel")
+    ap.add_argument("--kv-split", type=int, default=0, help="override the workload's kv_split (experiments)")
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -70,7 +71,7 @@ def main():
     wl_cpu = fd.utils.make_config5_bf16_twin() if args.bf16_twin else fd.utils.make_config(args.config)
     wl = wl_cpu.to(dev)
     B, Hq, D = wl.q.shape
-    S = wl.kv_split
+    S = args.kv_split or wl.kv_split
     algo_bytes = wl_cpu.algorithmic_bytes()
 
     # independent KV pools: pool 0 holds the seeded data (checked against the CPU baseline), the

@@ -202,8 +202,8 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
  * the partial workspace is internal, fewer and longer splits mean fewer workgroup
  * prologues and fewer partials for the combine.  Returns min(params->num_splits, the split
- * count that (1) puts one wave on every wave slot of the chip and (2) keeps every
- * workgroup at or below 2048 tokens of a full-length sequence), or a negative fd_status.
+ * count that (1) reaches about 1024 waves with two waves per (KV head, split) and (2) keeps
+ * every split of a full-length sequence at or below 4096 tokens), or a negative fd_status.
  * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
  * params->num_splits splits with the reference's ranges.
  */

@@ -42,19 +42,36 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
   *shift = k;
 }
 
-// Waves per workgroup when the caller does not choose: enough waves to put
-// about 8 on every CU (256 CUs), but never more waves than 32-token tiles a
-// split can have.
-int choose_waves(int64_t workgroups, int64_t max_tokens_per_split, int tile) {
+// Launch-shape policy, from sweeps on one MI355X (256 CUs): the kernels stream best with about
+// 1024 waves in flight, each walking a long token range (every wave pays a fixed prologue /
+// epilogue, and every split adds a partial for the combine), and with at least one workgroup per CU.
+constexpr int64_t kTargetWaves = 1024;
+constexpr int64_t kMinWorkgroups = 256;
+constexpr int64_t kMaxTokensPerSplit = 4096;   // keeps a ragged batch balanceable by the dispatcher
+
+// Waves per (KV head, split) when the caller does not choose: the smallest power of two that reaches
+// kTargetWaves, never more waves than tiles a split can have.
+int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile) {
   int64_t tiles = (max_tokens_per_split + tile - 1) / tile;
   int w = 1;
-  while (w < 8 && workgroups * w < 2048 && w * 2 <= tiles) w *= 2;
+  while (w < 8 && head_splits * w < kTargetWaves && w * 2 <= tiles) w *= 2;
   const char* env = getenv("FD_WAVES_PER_BLOCK");
   if (env) {
     int e = atoi(env);
     if (e == 1 || e == 2 || e == 4 || e == 8) w = e;
   }
   return w;
+}
+
+// Adjacent KV heads per workgroup (one wave each): sibling waves fetch up to 512 contiguous bytes of
+// every token row together.  Bounded by 8 waves per workgroup and by keeping one workgroup per CU.
+int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_splits) {
+  int h = row_bytes > 0 ? 512 / row_bytes : 1;
+  const char* env = getenv("FD_HEADS_PER_BLOCK");
+  if (env && atoi(env) > 0) h = atoi(env);
+  if (h < 1) h = 1;
+  while (h > 1 && (kv_heads % h != 0 || h * waves > 8 || head_splits / h < kMinWorkgroups)) h >>= 1;
+  return h;
 }
 
 }  // namespace
@@ -75,11 +92,6 @@ struct FusedTail {          // what the fused combine needs on top of the split 
   int64_t stride_obs = 0, stride_oh = 0;
   int32_t num_extra = 0, lse_column = 0;
 };
-
-// fd_plan_splits: wave slots of one MI355X at the split kernels' occupancy (256 CUs x 4 SIMDs x 2 waves) and the
-// largest token count one workgroup should own (keeps a ragged batch balanceable by the dispatcher).
-constexpr int64_t kResidentWaves = 2048;
-constexpr int64_t kMaxTokensPerGroup = 2048;
 
 // Largest dynamic LDS a workgroup may ask for on gfx950 (160 KB per CU).
 constexpr size_t kMaxLds = 160 * 1024;
@@ -172,20 +184,10 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
   const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
   int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
-  // Adjacent KV heads per workgroup (one wave each): sibling waves then fetch up to 512 contiguous bytes
-  // of every token row together.  Only the MFMA kernels, and not with the fused combine (its tickets
-  // are per KV head).
+  // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
-  if (use_mfma && !fuse) {
-    const int row_bytes = D * kvsz;
-    int h = 512 / row_bytes;
-    const char* env = getenv("FD_HEADS_PER_BLOCK");
-    if (env && atoi(env) > 0) h = atoi(env);
-    while (h > 1 && (a.Hkv % h != 0 || h * waves > 8)) h >>= 1;
-    if (h < 1) h = 1;
-    a.hpw = h;
-  }
+  if (use_mfma && !fuse) a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs);
   waves *= a.hpw;   // total waves of a workgroup
 
   // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS
@@ -265,12 +267,12 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   const bool mfma = p->head_dim == 128 && G >= 4 && (G <= 16 || G % 16 == 0) && p->path != FD_PATH_VALU &&
                     (p->kv_dtype == FD_FP8_E4M3 || p->kv_dtype == FD_F16 || p->kv_dtype == FD_BF16);
   const int64_t nhb = mfma ? (G + 15) / 16 : (G + (G >= 3 ? 4 : G) - 1) / (G >= 3 ? 4 : G);
-  const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // workgroups per split
+  const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
-  // (1) enough splits to put one wave on every wave slot of the chip (256 CUs x 8 waves) ...
-  int64_t s_fill = (kResidentWaves + groups - 1) / groups;
-  // (2) ... and enough that no workgroup owns more than kMaxTokensPerGroup tokens of a full-length sequence
-  int64_t s_bal = (max_tokens + kMaxTokensPerGroup - 1) / kMaxTokensPerGroup;
+  // (1) enough splits to reach the target wave count with two waves per head-split ...
+  int64_t s_fill = (kTargetWaves + 2 * groups - 1) / (2 * groups);
+  // (2) ... and enough that no split of a full-length sequence is longer than kMaxTokensPerSplit
+  int64_t s_bal = (max_tokens + kMaxTokensPerSplit - 1) / kMaxTokensPerSplit;
   int64_t s = s_fill > s_bal ? s_fill : s_bal;
   if (s > p->num_splits) s = p->num_splits;
   if (s < 1) s = 1;
