@@ -113,6 +113,11 @@ __device__ __forceinline__ float fd_softcap(float x, float cap, float inv_cap) {
   return cap * (1.0f - 2.0f / (1.0f + e));
 }
 
+// K/V rows are read exactly once per decode step: non-temporal loads keep them from being allocated in the
+// caches on their way through (measured with a pure-read probe on the same access pattern: 6.97 vs 6.15 TB/s).
+__device__ __forceinline__ u32x4 load_stream_b128(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+__device__ __forceinline__ u32x2 load_stream_b64(const void* p) { return __builtin_nontemporal_load((const u32x2*)p); }
+
 // Orders LDS accesses of one wave: lanes of a wave exchange data through LDS
 // without a workgroup barrier (the LDS queue of a wave is in order); this only
 // stops the compiler from moving accesses across the point.

@@ -108,11 +108,11 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
   };
   auto issue_k = [&]() {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) kraw[i] = *(const u32x4*)(kbase + (int64_t)rows[i] * k_pitch);
+    for (int i = 0; i < 8; ++i) kraw[i] = load_stream_b128(kbase + (int64_t)rows[i] * k_pitch);
   };
   auto issue_v = [&]() {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) vraw[i] = *(const u32x4*)(vbase + (int64_t)rows[i] * v_pitch);
+    for (int i = 0; i < 8; ++i) vraw[i] = load_stream_b128(vbase + (int64_t)rows[i] * v_pitch);
   };
 
   float m = -INFINITY;  // running max of head c (identical in the 4 wave rows)

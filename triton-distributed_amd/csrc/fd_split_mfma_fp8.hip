@@ -94,14 +94,14 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int row = __shfl(rv, 8 * i + (lane >> 3));
-      kraw[i] = *(const u32x4*)(kbase + (int64_t)row * k_pitch);
+      kraw[i] = load_stream_b128(kbase + (int64_t)row * k_pitch);
     }
   };
   auto issue_v = [&](int rv, int kblk) {  // the 8 rows of P.V block kblk
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int row = __shfl(rv, 16 * (2 * kblk + (e >> 2)) + 4 * g + (e & 3));
-      vraw[8 * kblk + e] = *(const u32x2*)(vbase + (int64_t)row * v_pitch);
+      vraw[8 * kblk + e] = load_stream_b64(vbase + (int64_t)row * v_pitch);
     }
   };
 

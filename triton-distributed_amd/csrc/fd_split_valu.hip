@@ -137,8 +137,8 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = __shfl(rv, u * TPI + rg);
-      kraw[u] = *(const u32x4*)(kbase + (int64_t)row * k_pitch);
-      vraw[u] = *(const u32x4*)(vbase + (int64_t)row * v_pitch);
+      kraw[u] = load_stream_b128(kbase + (int64_t)row * k_pitch);
+      vraw[u] = load_stream_b128(vbase + (int64_t)row * v_pitch);
     }
   };
   if (t0 < t1) {
