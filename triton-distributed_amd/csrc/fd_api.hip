@@ -219,6 +219,12 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
 extern "C" {
 
+static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
+                        const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials,
+                        int64_t stride_mid_ob, int64_t stride_mid_oh, int64_t stride_mid_os, int64_t stride_obs,
+                        int64_t stride_oh, int32_t mode, const void* extra_out, const float* extra_lse,
+                        int32_t num_extra, const fd_params* p, bool all_slots_written);
+
 int fd_split_kv(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out_split,
                 float* lse_split, float sm_scale, const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
                 int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok, int64_t stride_k_h,
@@ -253,9 +259,9 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
                       batch, stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_o_bs,
                       stride_o_h, stride_o_split, stride_table_bs, seq_order, p, &tail, &fused);
   if (rc != FD_OK || fused || batch == 0) return rc;
-  return fd_combine(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
-                    stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out, extra_lse,
-                    num_extra, p);
+  return combine_impl(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
+                      stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out,
+                      extra_lse, num_extra, p, true);
 }
 
 int fd_plan_splits(const fd_params* p, int32_t batch) {
@@ -279,10 +285,11 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   return (int)s;
 }
 
-int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
-               const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials, int64_t stride_mid_ob,
-               int64_t stride_mid_oh, int64_t stride_mid_os, int64_t stride_obs, int64_t stride_oh, int32_t mode,
-               const void* extra_out, const float* extra_lse, int32_t num_extra, const fd_params* p) {
+static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
+                        const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials,
+                        int64_t stride_mid_ob, int64_t stride_mid_oh, int64_t stride_mid_os, int64_t stride_obs,
+                        int64_t stride_oh, int32_t mode, const void* extra_out, const float* extra_lse,
+                        int32_t num_extra, const fd_params* p, bool all_slots_written) {
   if (!p) return fail(FD_ERR_INVALID_ARG, "fd_combine: params is NULL");
   if (!mid_o || !out || !seqlens) return fail(FD_ERR_INVALID_ARG, "fd_combine: NULL tensor pointer");
   if (batch < 0 || q_heads <= 0 || num_partials <= 0 || num_extra < 0)
@@ -308,9 +315,19 @@ int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out,
   a.mode = mode; a.mid_dtype = p->mid_dtype; a.out_dtype = p->out_dtype;
   a.vec_mid = (p->mid_dtype == FD_F32 && aligned16(mid_o) && stride_mid_ob % 4 == 0 && stride_mid_oh % 4 == 0 &&
                stride_mid_os % 4 == 0) ? 1 : 0;
+  a.all_slots_written = all_slots_written ? 1 : 0;
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;
+}
+
+int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
+               const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials, int64_t stride_mid_ob,
+               int64_t stride_mid_oh, int64_t stride_mid_os, int64_t stride_obs, int64_t stride_oh, int32_t mode,
+               const void* extra_out, const float* extra_lse, int32_t num_extra, const fd_params* p) {
+  return combine_impl(stream, mid_o, mid_lse, out, lse_out, seqlens, batch, q_heads, num_partials, stride_mid_ob,
+                      stride_mid_oh, stride_mid_os, stride_obs, stride_oh, mode, extra_out, extra_lse, num_extra, p,
+                      false);
 }
 
 int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* seq_order) {

@@ -113,6 +113,71 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   }
 }
 
+// Few partials (<= kSmallMax), fp32 and 128-bit aligned, produced by this library's split kernel in the
+// same call: every slot is written (an empty split holds out = 0, lse = -inf), so validity needs no
+// kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which leaves one
+// dependent memory round trip.  Thread (r, c): partial r (and r + ROWS), 128-bit column chunk c.
+constexpr int kSmallMax = 16;
+
+template <int D>
+__global__ void __launch_bounds__(kCombineThreads) fd_combine_small_kernel(const CombineArgs a) {
+  constexpr int CG = D / 4;
+  constexpr int ROWS = kCombineThreads / CG;
+  __shared__ __align__(16) float s_acc[ROWS][D];
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x / a.Hq;
+  const int h = blockIdx.x - b * a.Hq;
+  const int S = a.num_partials;
+  const float* mid = (const float*)a.mid_o + (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
+  const int r = tid / CG;
+  const int c = tid - r * CG;
+  constexpr int PASSES = (kSmallMax + ROWS - 1) / ROWS;
+  f32x4 o[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int s = r + p * ROWS;
+    o[p] = s < S ? *(const f32x4*)(mid + (int64_t)s * a.s_ms + 4 * c) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  float lse[kSmallMax];
+#pragma unroll
+  for (int s = 0; s < kSmallMax; ++s) {
+    lse[s] = -INFINITY;
+    if (s < S) lse[s] = a.mid_lse ? a.mid_lse[((int64_t)b * a.Hq + h) * S + s] : mid[(int64_t)s * a.s_ms + D];
+  }
+  float M = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kSmallMax; ++s) M = fmaxf(M, lse[s]);
+  float L = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int s = 0; s < kSmallMax; ++s) L += __expf(lse[s] - M);   // exp(-inf) = 0 for empty / absent splits
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const int s = r + p * ROWS;
+      float wgt = 0.f;
+#pragma unroll
+      for (int q = 0; q < kSmallMax; ++q) wgt = q == s ? __expf(lse[q] - M) : wgt;
+      acc += o[p] * wgt;
+    }
+  }
+  *(f32x4*)&s_acc[r][4 * c] = acc;
+  __syncthreads();
+  if (tid < D) {
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) v += s_acc[i][tid];
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
+    store_from_f32(a.out, out_base + tid, a.out_dtype, v * inv);
+    if (tid == 0) {
+      const float res = L > 0.f ? M + __logf(L) : -INFINITY;
+      if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, res);
+      if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = res;
+    }
+  }
+}
+
 // order[rank] = sequence index, sequences ranked by kv_len descending, ties by index.
 __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restrict__ kv_lens, int batch,
                                                           int32_t* __restrict__ order) {
@@ -132,10 +197,12 @@ __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restr
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a) {
   const unsigned grid = (unsigned)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
+  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 &&
+                     a.num_partials <= kSmallMax && a.mid_dtype == FD_F32 && a.vec_mid;
   switch (a.D) {
-    case 64: kern = fd_combine_kernel<64>; break;
-    case 128: kern = fd_combine_kernel<128>; break;
-    case 256: kern = fd_combine_kernel<256>; break;
+    case 64: kern = small ? fd_combine_small_kernel<64> : fd_combine_kernel<64>; break;
+    case 128: kern = small ? fd_combine_small_kernel<128> : fd_combine_kernel<128>; break;
+    case 256: kern = small ? fd_combine_small_kernel<256> : fd_combine_kernel<256>; break;
     default: return FD_ERR_UNSUPPORTED;
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
