@@ -211,6 +211,18 @@ def main():
                      "traffic": traffic, "kernel_us": round(split_us, 3)},
     }
 
+    # MFMA work of the split kernel (secondary figure: the path is HBM-bound).  Issued flops follow from the tiling:
+    # per 32 tokens of one (sequence, KV head, block of <=16 query heads) 16 MFMAs of 16x16x32 (16 384 flop each);
+    # the committed counter run (profiles/*mfma_utilisation.md) reads exactly this number.
+    G = Hq // wl.k_cache.shape[2]
+    if D == 128 and G >= 4 and args.path != "valu" and wl.q.dtype != torch.float32:
+        tokens = int(wl_cpu.kv_lens.sum())
+        nhb = -(-G // 16)
+        issued = tokens * wl.k_cache.shape[2] * nhb * 16 * 16384 / 32
+        result["mfma"] = {"useful_flop_per_step": wl_cpu.flops(), "issued_flop_per_step": int(issued),
+                          "issued_tflops": round(issued / (split_us * 1e-6) / 1e12, 1),
+                          "frac_of_dense_bf16_peak": round(issued / (split_us * 1e-6) / 2.5e15, 4)}
+
     if not args.no_cpu_baseline:
         import oracle  # the checker, timed as the CPU baseline only
         n_seq = args.cpu_seqs or (B if algo_bytes < 6e8 else max(1, min(B, 4)))
