@@ -105,8 +105,13 @@ def check(status: int) -> None:
         raise RuntimeError(f"flash_decode library error {status}: {msg}")
 
 
-def stream_handle(stream=None) -> int:
-    """hipStream_t of ``stream`` (a torch stream) or of the current torch stream."""
-    if stream is None:
-        stream = torch.cuda.current_stream()
-    return stream.cuda_stream
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def stream_handle(stream=None, device_index=None) -> int:
+    """hipStream_t of ``stream`` (a torch stream) or of the current torch stream of the device."""
+    if stream is not None:
+        return stream.cuda_stream
+    if _raw_stream is not None:   # a direct lookup: torch.cuda.current_stream() costs several microseconds
+        return _raw_stream(torch.cuda.current_device() if device_index is None else device_index)
+    return torch.cuda.current_stream().cuda_stream

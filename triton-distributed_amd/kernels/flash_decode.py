@@ -82,7 +82,8 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
     assert kv_lens.dtype == torch.int32 and kv_lens.is_contiguous()
     if out is None:
         out = torch.empty_like(kv_lens)
-    check(lib.fd_schedule(stream_handle(stream), kv_lens.data_ptr(), kv_lens.numel(), out.data_ptr()))
+    check(lib.fd_schedule(stream_handle(stream, kv_lens.device.index), kv_lens.data_ptr(), kv_lens.numel(),
+                          out.data_ptr()))
     return out
 
 
@@ -126,39 +127,51 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         raise RuntimeError("k_scale and v_scale must be given together")
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
     lib = load_library()
-    hstream = stream_handle(stream)
+    hstream = stream_handle(stream, q.device.index)
 
-    lse_split = None
+    # Partials.  Internal ones are fp32 [B,Hq,S,Dv] + LSE [B,Hq,S] addressed by raw pointers (no tensor views
+    # on the hot path); a caller-supplied buffer keeps the reference layout [B,Hq,S,Dv+1].
     if output_split is None:
         if plan_splits:
             # nobody looks at the partials: let the library merge splits (fewer, longer ones)
-            plan = _make_params(q, k_cache, block_table, num_splits, soft_cap, FD_F32, FD_F32, k_scale, v_scale, path,
-                                waves_per_block)
-            num_splits = lib.fd_plan_splits(byref(plan), batch)
-            if num_splits < 0:
-                check(num_splits)
-        # internal partials: fp32, 128-bit aligned rows, LSE in its own buffer
+            key = (batch, q_heads, kv_heads, q_head_dim, page_size, num_splits, block_table.shape[1], k_cache.dtype,
+                   k_scale is not None, path)
+            planned = _PLAN_CACHE.get(key)
+            if planned is None:
+                plan = _make_params(q, k_cache, block_table, num_splits, soft_cap, FD_F32, FD_F32, k_scale, v_scale,
+                                    path, waves_per_block)
+                planned = lib.fd_plan_splits(byref(plan), batch)
+                if planned < 0:
+                    check(planned)
+                _PLAN_CACHE[key] = planned
+            num_splits = planned
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
         if (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
                 and workspace.is_contiguous() and workspace.numel() >= n_o + n_l):
             # a float32 workspace that is large enough holds the partials: no allocation in the call
-            flat = workspace.view(-1)
-            output_split = flat[:n_o].view(batch, q_heads, num_splits, v_head_dim)
-            lse_split = flat[n_o:n_o + n_l].view(batch, q_heads, num_splits)
+            hold = workspace
         else:
-            output_split = torch.empty([batch, q_heads, num_splits, v_head_dim], dtype=torch.float32, device=q.device)
-            lse_split = torch.empty([batch, q_heads, num_splits], dtype=torch.float32, device=q.device)
+            hold = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
+            if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
+                hold.record_stream(stream)
+        mid_ptr = hold.data_ptr()
+        lse_split_ptr = mid_ptr + 4 * n_o
+        mid_dtype = FD_F32
+        so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
     else:
         assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
+        assert output_split.shape[2] == num_splits
+        mid_ptr, lse_split_ptr, mid_dtype = output_split.data_ptr(), None, fd_dtype_of(output_split)
+        so_b, so_h, so_s = output_split.stride(0), output_split.stride(1), output_split.stride(2)
     out_cols = v_head_dim + 1 if with_lse_column else v_head_dim
     if output_combine is None:
         output_combine = torch.empty([batch, q_heads, out_cols], dtype=q.dtype, device=q.device)
     else:
         assert output_combine.shape[-1] >= out_cols and output_combine.stride(-1) == 1
 
-    p = _make_params(q, k_cache, block_table, num_splits, soft_cap, fd_dtype_of(output_split),
-                     fd_dtype_of(output_combine), k_scale, v_scale, path, waves_per_block)
+    p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
+                     v_scale, path, waves_per_block)
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:
@@ -172,19 +185,19 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
     tickets = _tickets(q.device, hstream, batch * q_heads) if fuse_combine else None
     check(lib.fd_decode(
-        hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_split.data_ptr(),
-        lse_split.data_ptr() if lse_split is not None else None, output_combine.data_ptr(),
-        lse_out.data_ptr() if lse_out is not None else None, float(scale), block_table.data_ptr(),
-        kv_lens.data_ptr(), batch,
+        hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), mid_ptr, lse_split_ptr,
+        output_combine.data_ptr(), lse_out.data_ptr() if lse_out is not None else None, float(scale),
+        block_table.data_ptr(), kv_lens.data_ptr(), batch,
         q.stride(0), q.stride(1), k_cache.stride(-3), k_cache.stride(-2), v_cache.stride(-3), v_cache.stride(-2),
-        output_split.stride(0), output_split.stride(1), output_split.stride(2), block_table.stride(0),
-        output_combine.stride(0), output_combine.stride(1),
+        so_b, so_h, so_s, block_table.stride(0), output_combine.stride(0), output_combine.stride(1),
         seq_order.data_ptr() if seq_order is not None else None,
         FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
         ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra,
         tickets.data_ptr() if tickets is not None else None, byref(p)))
     return output_combine
 
+
+_PLAN_CACHE = {}   # fd_plan_splits results by problem shape
 
 # Zero-initialised ticket counters of the fused combine, one buffer per (device, stream): calls on
 # different streams may overlap and must not share counters; the kernels leave them at zero.
@@ -276,7 +289,7 @@ def _inter_rank_launch(Mid_O, o, B_Seqlens, batch, q_heads, stride_mid_ob, strid
     p.mid_dtype = fd_dtype_of(Mid_O)
     p.out_dtype = fd_dtype_of(o)
     check(lib.fd_combine(
-        stream_handle(stream), Mid_O.data_ptr(), None, o.data_ptr(),
+        stream_handle(stream, o.device.index), Mid_O.data_ptr(), None, o.data_ptr(),
         lse_out.data_ptr() if lse_out is not None else None, B_Seqlens.data_ptr(), batch, q_heads, NUM_KV_SPLITS,
         stride_mid_ob, stride_mid_oh, stride_mid_os, stride_obs, stride_oh, FD_COMBINE_RANK, None, None, 0, byref(p)))
     return o
