@@ -400,3 +400,49 @@ def test_errors_are_reported_not_fatal(fd):
     out = fd.gqa_fwd_batch_decode(wl.q, wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, wl.scale)
     torch.cuda.synchronize()
     assert torch.isfinite(out).all()
+
+
+# ---- HIP graph capture: the whole step (scheduler + split + combine) replays from a graph
+@pytest.mark.parametrize("variant", ["plain", "persistent"])
+def test_graph_capture_and_replay(fd, variant):
+    wl = _grid_workload(fd, [1320, 463, 2049, 77], (32, 8), 128, 16, torch.bfloat16, 0, seed=81).to(DEV)
+    B = 4
+    out = torch.empty(B, 32, 128, dtype=torch.bfloat16, device=DEV)
+    lse = torch.empty(B, 32, dtype=torch.float32, device=DEV)
+    ws = torch.empty(B * 32 * 32 * 129, dtype=torch.float32, device=DEV)
+    order = torch.empty(B, dtype=torch.int32, device=DEV)
+    fn = fd.gqa_fwd_batch_decode_persistent if variant == "persistent" else fd.gqa_fwd_batch_decode
+
+    def step():
+        kw = {}
+        if variant == "persistent":
+            fd.schedule_sequences(wl.kv_lens, out=order)
+            kw["seq_order"] = order
+        fn(wl.q, wl.k_cache, wl.v_cache, ws, [1] * B, wl.kv_lens, wl.block_table, wl.scale, 0.0,
+           output_combine=out, kv_split=32, lse_out=lse, **kw)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    for it in range(4):
+        # new query and new lengths, written in place (the graph holds the addresses)
+        wl.q.copy_(torch.randn(wl.q.shape, generator=gen).to(torch.bfloat16))
+        wl.kv_lens.copy_(torch.tensor([1320 - 100 * it, 463 + it, 2049 - 500 * it, 77 + 9 * it], dtype=torch.int32))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_out, got_lse = out.clone(), lse.clone()
+        out.zero_()
+        lse.zero_()
+        step()                                   # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(got_out, out) and torch.equal(got_lse, lse), f"replay {it} differs from eager"
+    ref, ref_lse = oracle_decode(wl.to("cpu"))
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)

@@ -163,3 +163,28 @@ def test_sp_layer_staging_ring_grows_and_shrinks(fd):
     assert layer.max_allgather_buffer_size == base
     layer.finalize()
     assert layer.ag_buffer is None
+
+
+def test_split_plan_policy(fd):
+    """fd_plan_splits: an upper-bounded split count from host-known sizes only (no kv_lens read)."""
+    import ctypes
+    lib = fd.load_library()
+    L = fd._lib
+
+    def plan(B, Hq, Hkv, S, max_pages, P=16, kv=L.FD_BF16, D=128):
+        p = L.FdParams()
+        p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits = Hq, Hkv, D, P, S
+        p.num_pages, p.max_pages_per_seq, p.q_dtype, p.kv_dtype = 10, max_pages, L.FD_BF16, kv
+        return lib.fd_plan_splits(ctypes.byref(p), B)
+
+    assert plan(8, 32, 8, 32, 512) == 8            # config 2: 1024 waves with 2 waves per (head, split)
+    assert plan(1, 32, 8, 32, 8192) == 32          # config 3: one sequence, all the splits the caller allows
+    assert plan(64, 32, 8, 32, 2048) == 8          # config 4: <= 4096 tokens per split of a full-length sequence
+    assert plan(32, 64, 8, 64, 1024, kv=L.FD_FP8_E4M3) == 4
+    assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
+    assert plan(4096, 32, 8, 32, 1) == 1
+    for args in [(3, 16, 16, 32, 83), (7, 6, 1, 5, 1000), (2, 64, 8, 64, 100000)]:
+        got = plan(*args)
+        assert 1 <= got <= args[3]
+    assert plan(0, 32, 8, 32, 512) < 0 and b"fd_plan_splits" in lib.fd_last_error()
+    assert lib.fd_plan_splits(None, 1) < 0
