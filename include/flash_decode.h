@@ -209,6 +209,55 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  */
 FD_API int fd_plan_splits(const fd_params* params, int32_t batch);
 
+/*
+ * Rotary position embedding applied on the way into the cache, as the reference's
+ * apply_rotary_pos_emb does right before its cache update
+ * (python/triton_dist/layers/amd/tp_attn.py:72-125 kernel, :128-160 launch, :232-241 and
+ * :263-264 call sites): out[i] = x[i]*cos[i] - x[i+D/2]*sin[i],
+ * out[i+D/2] = x[i+D/2]*cos[i] + x[i]*sin[i] for i < D/2, in fp32, each product and sum
+ * rounded separately, the result rounded to the activation dtype.
+ */
+typedef struct fd_rope {
+  const float* cos_sin;       /* [max_positions, D] fp32: D/2 cosines then D/2 sines per row
+                                 (tp_attn.py:62-69), 16-byte aligned rows                  */
+  int64_t stride_cos_sin;     /* row stride in elements                                    */
+  const void* position_ids;   /* [batch, new_tokens]                                       */
+  int32_t position_dtype;     /* 0: int32, 1: int64                                        */
+  int32_t max_positions;      /* positions are clamped into [0, max_positions)             */
+  int64_t stride_pos_b, stride_pos_t;
+  const void* q;              /* NULL, or [batch, new_tokens, Hq, D] in params->q_dtype     */
+  void* q_out;                /* rotated q, same dtype; may be q itself                    */
+  int64_t stride_q_b, stride_q_t, stride_q_h;
+  int64_t stride_qo_b, stride_qo_t, stride_qo_h;
+} fd_rope;
+
+/*
+ * The step before the decode: appends `new_tokens` tokens of K and V per sequence to the
+ * paged pool at logical positions kv_lens[b] .. kv_lens[b]+new_tokens-1, converting from the
+ * activation dtype (params->q_dtype) to the cache dtype (params->kv_dtype; FD_FP8_E4M3 stores
+ * clamp(x / scale[kv head], +-448) rounded to nearest even, with params->k_scale / v_scale).
+ * The pool layout [num_pages, P, Hkv, D] with an int32 block table is the one the decode
+ * reads (python/triton_dist/test/nvidia/test_decode_attn.py:150-156); the reference itself
+ * only has a dense cache whose update is a slice assignment
+ * (python/triton_dist/models/kv_cache.py:43-50, called at layers/amd/tp_attn.py:265), which
+ * is this layout with one page per sequence.  With `rope`, K is rotated before it is stored
+ * and, if rope->q is given, Q is rotated in the same launch.
+ *
+ *  k_new, v_new  [batch, new_tokens, Hkv, D], element strides stride_*n_b / _t / _h, last dim
+ *                contiguous, 16-byte aligned rows.  Both NULL: only rope->q is processed.
+ *  kv_lens       [batch] tokens already in the cache (not modified)
+ *  kv_lens_out   NULL, or [batch] (not kv_lens itself): min(kv_lens[b] + new_tokens, capacity)
+ *  A token whose position is at or beyond max_pages_per_seq * page_size is not written.
+ */
+FD_API int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                 const int32_t* block_table, const int32_t* kv_lens, int32_t* kv_lens_out,
+                 int32_t batch, int32_t new_tokens,
+                 int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
+                 int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h,
+                 int64_t stride_k_tok, int64_t stride_k_h,
+                 int64_t stride_v_tok, int64_t stride_v_h,
+                 int64_t stride_table_bs, const fd_rope* rope, const fd_params* params);
+
 /* Message for the last non-zero status returned on this thread ("" if none). */
 FD_API const char* fd_last_error(void);
 

@@ -13,6 +13,13 @@ from .ref_decode import (  # noqa: F401
     dequant_fp8_cache,
     quantize_fp8_cache,
 )
+from .ref_kv_append import (  # noqa: F401
+    ref_set_cos_sin_cache,
+    ref_rope,
+    ref_quantize_fp8,
+    brute_force_fp8,
+    ref_kv_append,
+)
 from .split_combine_model import (  # noqa: F401
     split_range,
     model_split_kv,

@@ -373,3 +373,127 @@ def test_fp8_quantise_dequantise_round_trip():
     assert (err <= bound * 1.0001).all()
     # the largest element of every head maps to +-448 exactly
     assert torch.equal(back.abs().amax(dim=(0, 1, 3)), scale * 448.0)
+
+
+# ------------------------------------------------------------------ write side: rotary + cache update
+
+def test_cos_sin_table_definition():
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, 8, 2, dtype=torch.float32) / 8))   # D = 8: 4 frequencies
+    tab = oracle.ref_set_cos_sin_cache(inv_freq, 16)
+    assert tab.shape == (16, 8)
+    assert torch.equal(tab[0], torch.tensor([1.0] * 4 + [0.0] * 4))                    # angle 0
+    # row t: first half cos(t * f_i), second half sin(t * f_i); f_0 = 1, f_1 = 10000^(-1/4) = 0.1
+    assert abs(float(tab[3, 0]) - math.cos(3.0)) < 1e-6 and abs(float(tab[3, 4]) - math.sin(3.0)) < 1e-6
+    assert abs(float(tab[5, 1]) - math.cos(0.5)) < 1e-6 and abs(float(tab[5, 5]) - math.sin(0.5)) < 1e-6
+
+
+def test_rope_is_complex_rotation():
+    g = torch.Generator().manual_seed(5)
+    B, T, H, D = 2, 3, 4, 16
+    x = torch.randn(B, T, H, D, generator=g)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    tab = oracle.ref_set_cos_sin_cache(inv_freq, 64)
+    pos = torch.randint(0, 64, (B, T), generator=g)
+    got = oracle.ref_rope(x, tab, pos).double()
+    # independent: element pair (i, i + D/2) is the complex number x1 + j x2, multiplied by exp(j * pos * f_i)
+    z = torch.complex(x[..., :D // 2].double(), x[..., D // 2:].double())
+    ang = pos.double()[:, :, None, None] * inv_freq.double()
+    zr = z * torch.exp(1j * ang)
+    want = torch.cat([zr.real, zr.imag], dim=-1)
+    assert (got - want).abs().max() < 1e-5
+    # a swapped sign or half would break the norm or the identity at angle 0
+    assert torch.allclose(got.norm(dim=-1), x.double().norm(dim=-1), atol=1e-5)
+    assert torch.equal(oracle.ref_rope(x, tab, torch.zeros(B, T, dtype=torch.long)), x)
+    # angles add: rotating by p then by q (second table row as a fresh rotation) equals rotating by p + q
+    p1, p2 = torch.full((B, T), 7), torch.full((B, T), 12)
+    twice = oracle.ref_rope(oracle.ref_rope(x, tab, p1), tab, p2)
+    once = oracle.ref_rope(x, tab, p1 + p2)
+    assert (twice - once).abs().max() < 1e-5
+    # out-of-table positions are clamped
+    assert torch.equal(oracle.ref_rope(x, tab, torch.full((B, T), 1000)), oracle.ref_rope(x, tab, torch.full((B, T), 63)))
+
+
+def test_rope_rounds_to_activation_dtype():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(1, 2, 2, 8, generator=g).to(torch.bfloat16)
+    tab = oracle.ref_set_cos_sin_cache(torch.tensor([1.0, 0.5, 0.25, 0.125]), 8)
+    got = oracle.ref_rope(x, tab, torch.tensor([[1, 5]]))
+    assert got.dtype == torch.bfloat16
+    want = oracle.ref_rope(x.float(), tab, torch.tensor([[1, 5]])).to(torch.bfloat16)
+    assert torch.equal(got, want)
+
+
+def test_fp8_rounding_against_brute_force_search():
+    g = np.random.default_rng(3)
+    tab = oracle.fp8_e4m3fn_decode_table()
+    finite = tab[~np.isnan(tab)]
+    mids = (np.sort(finite)[1:].astype(np.float64) + np.sort(finite)[:-1].astype(np.float64)) / 2   # every tie point
+    vals = np.concatenate([
+        g.normal(size=400) * 3, g.uniform(-448, 448, 300), g.uniform(-2 ** -6, 2 ** -6, 200),   # normals, subnormals
+        finite.astype(np.float64), mids, np.nextafter(mids.astype(np.float32), np.float32(1e9)).astype(np.float64),
+        np.nextafter(mids.astype(np.float32), np.float32(-1e9)).astype(np.float64), [0.0, 448.0, -448.0, 2 ** -10, 2 ** -9],
+    ]).astype(np.float32)
+    got = oracle.ref_quantize_fp8(torch.from_numpy(vals).view(-1, 1, 1), torch.ones(1)).view(-1).numpy()
+    want = oracle.brute_force_fp8(vals)
+    zero = vals == 0
+    assert np.array_equal(got[~zero], want[~zero])
+    assert np.all((got[zero] & 0x7F) == 0)
+    # scale divides, and values beyond the largest finite magnitude saturate instead of becoming NaN
+    q = oracle.ref_quantize_fp8(torch.tensor([[[1000.0, -1000.0, 3.0]]]), torch.tensor([2.0]))
+    assert q.view(-1).tolist() == [0x7E, 0xFE, int(oracle.brute_force_fp8(np.array([1.5], dtype=np.float32))[0])]
+
+
+@pytest.mark.parametrize("P", [1, 4, 16])
+def test_append_round_trip_through_gather(P):
+    from oracle.ref_decode import _gather_kv
+    g = torch.Generator().manual_seed(11 + P)
+    B, Hkv, D, num_pages = 3, 2, 8, 40
+    lens = [9, 1, 17]
+    maxp = max(-(-n // P) for n in lens)
+    perm = torch.randperm(num_pages, generator=g)
+    bt = torch.full((B, maxp), -7, dtype=torch.int32)
+    used = 0
+    for b, n in enumerate(lens):
+        need = -(-n // P)
+        bt[b, :need] = perm[used:used + need].to(torch.int32)
+        used += need
+    src_k = [torch.randn(n, Hkv, D, generator=g) for n in lens]
+    src_v = [torch.randn(n, Hkv, D, generator=g) for n in lens]
+    poison = 12345.0
+    kc = torch.full((num_pages, P, Hkv, D), poison)
+    vc = torch.full((num_pages, P, Hkv, D), poison)
+    cur = torch.zeros(B, dtype=torch.int32)
+    # append in ragged chunks: 1 token, then 3, then the rest one sequence at a time
+    for chunk in (1, 3, 100):
+        for b in range(B):
+            lo = int(cur[b])
+            hi = min(lo + chunk, lens[b])
+            if hi == lo:
+                continue
+            one_bt, one_len = bt[b:b + 1], cur[b:b + 1]
+            grown = oracle.ref_kv_append(src_k[b][lo:hi][None], src_v[b][lo:hi][None], kc, vc, one_bt, one_len)
+            assert int(grown[0]) == hi
+            cur[b] = hi
+    for b, n in enumerate(lens):
+        assert torch.equal(_gather_kv(kc, bt[b], n), src_k[b])
+        assert torch.equal(_gather_kv(vc, bt[b], n), src_v[b])
+    # exactly sum(lens) token rows were written, everything else still holds the poison
+    assert int((kc[..., 0, 0] != poison).sum()) == sum(lens) and int((vc[..., 0, 0] != poison).sum()) == sum(lens)
+
+
+def test_append_capacity_and_fp8():
+    g = torch.Generator().manual_seed(2)
+    P, Hkv, D = 4, 2, 8
+    bt = torch.tensor([[1, 0]], dtype=torch.int32)                    # capacity 8 tokens
+    kc = torch.zeros(3, P, Hkv, D, dtype=torch.uint8)
+    vc = torch.zeros(3, P, Hkv, D, dtype=torch.uint8)
+    k = torch.randn(1, 5, Hkv, D, generator=g)
+    v = torch.randn(1, 5, Hkv, D, generator=g)
+    ks, vs = torch.tensor([0.01, 0.02]), torch.tensor([0.03, 0.005])
+    grown = oracle.ref_kv_append(k, v, kc, vc, bt, torch.tensor([6], dtype=torch.int32), ks, vs)
+    assert int(grown[0]) == 8                                         # tokens 6, 7 stored, 8..10 dropped
+    assert torch.equal(kc[0, 2], oracle.ref_quantize_fp8(k[0, 0], ks)) and torch.equal(vc[0, 3], oracle.ref_quantize_fp8(v[0, 1], vs))
+    assert int(kc[2].sum()) == 0 and int(kc[1].sum()) == 0 and int(kc[0, :2].sum()) == 0
+    # dequantised values are within half an fp8 step (2^-4 relative) of the source
+    deq = oracle.dequant_fp8_cache(kc[0:1, 2:3], ks)[0, 0]
+    assert ((deq - k[0, 0]).abs() <= 0.0625 * k[0, 0].abs() + 0.01 * 2 ** -9 + 1e-7).all()

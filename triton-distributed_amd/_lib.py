@@ -24,8 +24,8 @@ FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_plan_splits", "fd_last_error",
-                    "fd_abi_version")
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_plan_splits", "fd_kv_append",
+                    "fd_last_error", "fd_abi_version")
 
 _DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
 if hasattr(torch, "float8_e4m3fn"):
@@ -50,6 +50,17 @@ class FdParams(Structure):
         ("q_dtype", c_int32), ("kv_dtype", c_int32), ("mid_dtype", c_int32), ("out_dtype", c_int32),
         ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
         ("path", c_int32), ("waves_per_block", c_int32),
+    ]
+
+
+class FdRope(Structure):
+    """Mirror of ``struct fd_rope``."""
+    _fields_ = [
+        ("cos_sin", c_void_p), ("stride_cos_sin", c_int64), ("position_ids", c_void_p),
+        ("position_dtype", c_int32), ("max_positions", c_int32), ("stride_pos_b", c_int64), ("stride_pos_t", c_int64),
+        ("q", c_void_p), ("q_out", c_void_p),
+        ("stride_q_b", c_int64), ("stride_q_t", c_int64), ("stride_q_h", c_int64),
+        ("stride_qo_b", c_int64), ("stride_qo_t", c_int64), ("stride_qo_h", c_int64),
     ]
 
 
@@ -86,6 +97,10 @@ def load_library(path: str = None) -> ctypes.CDLL:
         c_int32, c_void_p, POINTER(FdParams)]
     lib.fd_plan_splits.restype = c_int32
     lib.fd_plan_splits.argtypes = [POINTER(FdParams), c_int32]
+    lib.fd_kv_append.restype = c_int32
+    lib.fd_kv_append.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+        i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, POINTER(FdRope), POINTER(FdParams)]
     lib.fd_schedule.restype = c_int32
     lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]
     lib.fd_last_error.restype = c_char_p

@@ -330,6 +330,91 @@ int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out,
                       false);
 }
 
+int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                 const int32_t* block_table, const int32_t* kv_lens, int32_t* kv_lens_out, int32_t batch,
+                 int32_t new_tokens, int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
+                 int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h, int64_t stride_k_tok,
+                 int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_table_bs,
+                 const fd_rope* rope, const fd_params* p) {
+  const char* fn = "fd_kv_append";
+  if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
+  if (batch < 0 || new_tokens < 0) return fail(FD_ERR_INVALID_ARG, "%s: batch %d, new_tokens %d", fn, batch, new_tokens);
+  if (batch == 0 || new_tokens == 0) return FD_OK;
+  const bool append = k_new || v_new;
+  const bool with_q = rope && rope->q;
+  if (!append && !with_q) return fail(FD_ERR_INVALID_ARG, "%s: nothing to do (no k_new / v_new and no rope->q)", fn);
+  const int D = p->head_dim;
+  if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "%s: head_dim %d (64/128/256)", fn, D);
+  const int ssz = dtype_size(p->q_dtype);
+  if (!ssz || p->q_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: q_dtype %d", fn, p->q_dtype);
+  const int src16 = 16 / ssz;
+  if (p->q_heads <= 0 || p->kv_heads <= 0)
+    return fail(FD_ERR_INVALID_ARG, "%s: q_heads %d, kv_heads %d", fn, p->q_heads, p->kv_heads);
+
+  AppendArgs a;
+  memset(&a, 0, sizeof(a));
+  a.batch = batch; a.T = new_tokens; a.Hq = p->q_heads; a.Hkv = p->kv_heads; a.D = D;
+  int kv_dtype = p->q_dtype;
+  if (append) {
+    if (!k_new || !v_new || !k_cache || !v_cache || !block_table || !kv_lens)
+      return fail(FD_ERR_INVALID_ARG, "%s: NULL tensor pointer", fn);
+    if (kv_lens_out == kv_lens) return fail(FD_ERR_INVALID_ARG, "%s: kv_lens_out must not be kv_lens", fn);
+    if (p->page_size <= 0 || p->num_pages <= 0 || p->max_pages_per_seq <= 0)
+      return fail(FD_ERR_INVALID_ARG, "%s: page_size/num_pages/max_pages_per_seq must be > 0", fn);
+    if ((int64_t)p->num_pages * p->page_size >= (int64_t)1 << 31)
+      return fail(FD_ERR_TOO_LARGE, "%s: pool of %lld token rows exceeds 2^31", fn,
+                  (long long)p->num_pages * p->page_size);
+    if ((int64_t)p->max_pages_per_seq * p->page_size >= (int64_t)1 << 31)
+      return fail(FD_ERR_TOO_LARGE, "%s: block table capacity exceeds 2^31 tokens", fn);
+    kv_dtype = p->kv_dtype;
+    const int kvsz = dtype_size(kv_dtype);
+    if (!kvsz) return fail(FD_ERR_UNSUPPORTED, "%s: kv_dtype %d", fn, kv_dtype);
+    if (kv_dtype == FD_FP8_E4M3 && (!p->k_scale || !p->v_scale))
+      return fail(FD_ERR_INVALID_ARG, "%s: fp8 KV cache needs k_scale and v_scale", fn);
+    const int kv16 = 16 / kvsz;
+    if (!aligned16(k_cache) || !aligned16(v_cache) || stride_k_tok % kv16 || stride_k_h % kv16 ||
+        stride_v_tok % kv16 || stride_v_h % kv16)
+      return fail(FD_ERR_ALIGNMENT, "%s: K/V cache rows must be 16-byte aligned (pointer and token/head strides)", fn);
+    if (!aligned16(k_new) || !aligned16(v_new) || stride_kn_b % src16 || stride_kn_t % src16 || stride_kn_h % src16 ||
+        stride_vn_b % src16 || stride_vn_t % src16 || stride_vn_h % src16)
+      return fail(FD_ERR_ALIGNMENT, "%s: k_new / v_new rows must be 16-byte aligned (pointer and strides)", fn);
+    if (stride_k_tok <= 0 || stride_v_tok <= 0) return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
+    a.k_new = k_new; a.v_new = v_new; a.k_cache = k_cache; a.v_cache = v_cache;
+    a.bt = block_table; a.kv_lens = kv_lens; a.kv_lens_out = kv_lens_out;
+    a.k_scale = p->k_scale; a.v_scale = p->v_scale;
+    a.skn_b = stride_kn_b; a.skn_t = stride_kn_t; a.skn_h = stride_kn_h;
+    a.svn_b = stride_vn_b; a.svn_t = stride_vn_t; a.svn_h = stride_vn_h;
+    a.sk_t = stride_k_tok; a.sk_h = stride_k_h; a.sv_t = stride_v_tok; a.sv_h = stride_v_h;
+    a.sbt = stride_table_bs; a.P = p->page_size; a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
+  }
+  if (rope) {
+    if (!rope->cos_sin || !rope->position_ids) return fail(FD_ERR_INVALID_ARG, "%s: rope needs cos_sin and position_ids", fn);
+    if (rope->max_positions <= 0) return fail(FD_ERR_INVALID_ARG, "%s: rope->max_positions %d", fn, rope->max_positions);
+    if (rope->position_dtype != 0 && rope->position_dtype != 1)
+      return fail(FD_ERR_INVALID_ARG, "%s: rope->position_dtype %d (0: int32, 1: int64)", fn, rope->position_dtype);
+    if (!aligned16(rope->cos_sin) || rope->stride_cos_sin % 4 || rope->stride_cos_sin < D)
+      return fail(FD_ERR_ALIGNMENT, "%s: cos_sin rows must hold head_dim floats and be 16-byte aligned", fn);
+    a.cos_sin = rope->cos_sin; a.s_cs = rope->stride_cos_sin; a.pos = rope->position_ids;
+    a.pos_i64 = rope->position_dtype; a.max_pos = rope->max_positions;
+    a.sp_b = rope->stride_pos_b; a.sp_t = rope->stride_pos_t;
+    if (with_q) {
+      if (!rope->q_out) return fail(FD_ERR_INVALID_ARG, "%s: rope->q without rope->q_out", fn);
+      if (!aligned16(rope->q) || !aligned16(rope->q_out) || rope->stride_q_b % src16 || rope->stride_q_t % src16 ||
+          rope->stride_q_h % src16 || rope->stride_qo_b % src16 || rope->stride_qo_t % src16 ||
+          rope->stride_qo_h % src16)
+        return fail(FD_ERR_ALIGNMENT, "%s: q / q_out rows must be 16-byte aligned (pointer and strides)", fn);
+      a.q = rope->q; a.q_out = rope->q_out;
+      a.sq_b = rope->stride_q_b; a.sq_t = rope->stride_q_t; a.sq_h = rope->stride_q_h;
+      a.sqo_b = rope->stride_qo_b; a.sqo_t = rope->stride_qo_t; a.sqo_h = rope->stride_qo_h;
+    }
+  }
+  int rc = fd_launch_kv_append((hipStream_t)stream, a, p->q_dtype, kv_dtype);
+  if (rc == FD_ERR_LAUNCH) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
+  if (rc == FD_ERR_TOO_LARGE) return fail(rc, "%s: batch * new_tokens * heads too large for one launch", fn);
+  if (rc != FD_OK) return fail(rc, "%s: no kernel for q_dtype %d -> kv_dtype %d", fn, p->q_dtype, kv_dtype);
+  return FD_OK;
+}
+
 int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* seq_order) {
   if (!kv_lens || !seq_order) return fail(FD_ERR_INVALID_ARG, "fd_schedule: NULL pointer");
   if (batch < 0) return fail(FD_ERR_INVALID_ARG, "fd_schedule: batch = %d", batch);

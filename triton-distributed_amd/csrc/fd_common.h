@@ -70,6 +70,28 @@ struct CombineArgs {
                               // writes every slot (empty splits as out = 0, lse = -inf)
 };
 
+// Arguments of the KV-append / rotary kernel.
+struct AppendArgs {
+  const void* k_new;     // nullptr: no append (rotary of q only)
+  const void* v_new;
+  void* k_cache;
+  void* v_cache;
+  const int32_t* bt;
+  const int32_t* kv_lens;
+  int32_t* kv_lens_out;  // nullptr or [batch]
+  const float* k_scale;
+  const float* v_scale;
+  int64_t skn_b, skn_t, skn_h, svn_b, svn_t, svn_h, sk_t, sk_h, sv_t, sv_h, sbt;
+  int32_t batch, T, Hq, Hkv, D, P, max_pages, num_pages;
+  const float* cos_sin;  // nullptr: no rotation
+  const void* pos;       // [batch, T] int32 or int64
+  int64_t s_cs, sp_b, sp_t;
+  int32_t pos_i64, max_pos;
+  const void* q;         // nullptr: no query rows
+  void* q_out;
+  int64_t sq_b, sq_t, sq_h, sqo_b, sqo_t, sqo_h;
+};
+
 // ---------------------------------------------------------------- scalar conversions
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
@@ -357,3 +379,4 @@ int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype
 int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int waves);
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a);
 int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, int32_t* order);
+int fd_launch_kv_append(hipStream_t stream, const AppendArgs& a, int src_dtype, int kv_dtype);

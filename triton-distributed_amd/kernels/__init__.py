@@ -15,8 +15,18 @@ from .flash_decode import (  # noqa: F401
     get_triton_split_kv_algo_info,
     get_triton_combine_kv_algo_info,
 )
+from .kv_append import (  # noqa: F401
+    apply_rotary_pos_emb,
+    flash_attn_with_kvcache,
+    paged_kv_append,
+    rope_kv_append,
+)
 
 __all__ = [
+    "apply_rotary_pos_emb",
+    "flash_attn_with_kvcache",
+    "paged_kv_append",
+    "rope_kv_append",
     "get_triton_combine_kv_algo_info",
     "get_triton_split_kv_algo_info",
     "get_combine_kv_algo_info",

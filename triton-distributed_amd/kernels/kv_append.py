@@ -1,0 +1,208 @@
+"""Write side of the paged KV cache and the decode call that uses it.
+
+``rope_kv_append`` is one launch that does what the reference's decode block does in three
+steps right before attention (``python/triton_dist/layers/amd/tp_attn.py:262-265``): rotary
+embedding of Q, rotary embedding of K, and the cache update -- here an append into the
+paged pool ``[pages, P, Hkv, D]`` that the decode kernel reads, with fp8-e4m3 quantisation
+when the cache is fp8.  ``apply_rotary_pos_emb`` has the reference's signature
+(tp_attn.py:128-168).  ``flash_attn_with_kvcache`` is the call the reference's attention
+block makes (tp_attn.py:268-269, the flash-attn package's function), for one query token
+per sequence.
+
+Every function enqueues hand-written HIP kernels through the C ABI in
+``include/flash_decode.h``; there is no CPU path.
+"""
+from __future__ import annotations
+
+from ctypes import byref
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .._lib import FdParams, FdRope, check, fd_dtype_of, load_library, stream_handle
+from .flash_decode import _decode, _require_cuda
+
+
+def _rope_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdRope:
+    assert cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.stride(1) == 1
+    assert cos_sin.shape[1] == head_dim, "cos_sin rows hold head_dim/2 cosines then head_dim/2 sines"
+    assert position_ids.dim() == 2 and tuple(position_ids.shape) == (bsz, seq)
+    assert position_ids.dtype in (torch.int32, torch.int64)
+    r = FdRope()
+    r.cos_sin = cos_sin.data_ptr()
+    r.stride_cos_sin = cos_sin.stride(0)
+    r.position_ids = position_ids.data_ptr()
+    r.position_dtype = 1 if position_ids.dtype == torch.int64 else 0
+    r.max_positions = cos_sin.shape[0]
+    r.stride_pos_b, r.stride_pos_t = position_ids.stride(0), position_ids.stride(1)
+    return r
+
+
+def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
+                   kv_lens: Optional[torch.Tensor], *, kv_lens_out: Optional[torch.Tensor] = None,
+                   k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                   cos_sin: Optional[torch.Tensor] = None, position_ids: Optional[torch.Tensor] = None,
+                   q: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None, stream=None):
+    """Appends ``k_new`` / ``v_new`` ``[B, T, Hkv, D]`` at positions ``kv_lens[b] .. +T-1`` of the paged pool.
+
+    With ``cos_sin`` (fp32 ``[max_pos, D]``) and ``position_ids`` (``[B, T]`` int32/int64) K is rotated before it
+    is stored and ``q`` ``[B, T, Hq, D]`` (if given) is rotated into ``q_out`` (default: a new tensor; may be
+    ``q``) in the same launch.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
+    ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out`` (int32 ``[B]``, not ``kv_lens``) receives
+    the grown lengths.  Returns ``q_out`` (or ``None`` without ``q``).
+    """
+    lib = load_library()
+    append = k_new is not None
+    src = k_new if append else q
+    if src is None:
+        raise RuntimeError("rope_kv_append: neither k_new nor q given")
+    _require_cuda(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out, cos_sin, position_ids, q, q_out)
+    bsz, seq, _, head_dim = src.shape
+    p = FdParams()
+    p.head_dim = head_dim
+    p.q_dtype = fd_dtype_of(src)
+    p.q_heads = q.shape[2] if q is not None else 1
+    p.kv_heads = k_new.shape[2] if append else 1
+    ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+    skn = svn = (0, 0, 0)
+    sk = sv = (0, 0)
+    sbt = 0
+    if append:
+        assert v_new is not None and k_new.shape == v_new.shape and k_new.dtype == v_new.dtype
+        assert k_new.stride(-1) == 1 and v_new.stride(-1) == 1 and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+        assert k_cache.shape == v_cache.shape and k_cache.shape[2] == k_new.shape[2] and k_cache.shape[3] == head_dim
+        page_size = k_cache.shape[1]
+        assert k_cache.stride(0) == page_size * k_cache.stride(1) and v_cache.stride(0) == page_size * v_cache.stride(1)
+        assert block_table.dtype == torch.int32 and kv_lens.dtype == torch.int32 and block_table.stride(1) == 1
+        assert block_table.shape[0] == bsz and kv_lens.numel() == bsz and kv_lens.is_contiguous()
+        if (k_scale is None) != (v_scale is None):
+            raise RuntimeError("k_scale and v_scale must be given together")
+        if kv_lens_out is not None:
+            assert kv_lens_out.dtype == torch.int32 and kv_lens_out.is_contiguous() and kv_lens_out.numel() == bsz
+        p.page_size = page_size
+        p.num_pages = k_cache.shape[0]
+        p.max_pages_per_seq = block_table.shape[1]
+        p.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
+        p.k_scale, p.v_scale = ptr(k_scale), ptr(v_scale)
+        skn, svn = k_new.stride()[:3], v_new.stride()[:3]
+        sk, sv = (k_cache.stride(1), k_cache.stride(2)), (v_cache.stride(1), v_cache.stride(2))
+        sbt = block_table.stride(0)
+    rope = None
+    if cos_sin is not None:
+        rope = _rope_struct(cos_sin, position_ids, head_dim, bsz, seq)
+        if q is not None:
+            assert q.dim() == 4 and q.shape[0] == bsz and q.shape[1] == seq and q.shape[3] == head_dim
+            assert q.dtype == src.dtype and q.stride(-1) == 1
+            if q_out is None:
+                q_out = torch.empty_like(q)
+            assert q_out.shape == q.shape and q_out.dtype == q.dtype and q_out.stride(-1) == 1
+            rope.q, rope.q_out = q.data_ptr(), q_out.data_ptr()
+            rope.stride_q_b, rope.stride_q_t, rope.stride_q_h = q.stride()[:3]
+            rope.stride_qo_b, rope.stride_qo_t, rope.stride_qo_h = q_out.stride()[:3]
+    elif q is not None:
+        raise RuntimeError("rope_kv_append: q is only processed together with cos_sin / position_ids")
+    check(lib.fd_kv_append(
+        stream_handle(stream, src.device.index), ptr(k_new), ptr(v_new), ptr(k_cache), ptr(v_cache), ptr(block_table),
+        ptr(kv_lens), ptr(kv_lens_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
+        byref(rope) if rope is not None else None, byref(p)))
+    return q_out if q is not None else None
+
+
+def paged_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, *, kv_lens_out=None, k_scale=None,
+                    v_scale=None, stream=None):
+    """``rope_kv_append`` without the rotation: the plain cache update (models/kv_cache.py:43-50 for a paged pool)."""
+    rope_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out=kv_lens_out, k_scale=k_scale,
+                   v_scale=v_scale, stream=stream)
+
+
+def apply_rotary_pos_emb(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: torch.Tensor) -> torch.Tensor:
+    """Rotary embedding of ``x [bsz, seq, heads, head_dim]`` -> new tensor (tp_attn.py:128-168)."""
+    assert x.dim() == 4, "Input tensor x must be 4-dimensional"
+    assert position_ids.dim() == 2, "position_ids must be 2-dimensional"
+    x = x.contiguous()
+    return rope_kv_append(None, None, None, None, None, None, cos_sin=cos_sin.contiguous(),
+                          position_ids=position_ids, q=x)
+
+
+_ARANGE = {}
+
+
+def _dense_block_table(device, n):
+    key = (device.index, n)
+    t = _ARANGE.get(key)
+    if t is None:
+        t = torch.arange(n, dtype=torch.int32, device=device).view(n, 1)
+        _ARANGE[key] = t
+    return t
+
+
+def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None, rotary_sin=None,
+                            cache_seqlens: Union[int, torch.Tensor, None] = None, cache_batch_idx=None,
+                            cache_leftpad=None, block_table=None, softmax_scale=None, causal=False,
+                            window_size=(-1, -1), softcap=0.0, rotary_interleaved=True, alibi_slopes=None,
+                            num_splits=0, return_softmax_lse=False, *, cos_sin_cache=None, position_ids=None,
+                            k_scale=None, v_scale=None, kv_lens_out=None, stream=None, **decode_kw):
+    """Decode-step drop-in for the flash-attn call of the reference's attention block (tp_attn.py:268-269).
+
+    ``q [B, 1, Hq, D]``; ``k_cache`` / ``v_cache`` either dense ``[B_cache, L, Hkv, D]`` (the reference's
+    ``KV_Cache`` slice, models/kv_cache.py:36-44) or paged ``[pages, P, Hkv, D]`` with ``block_table``;
+    ``k`` / ``v [B, T, Hkv, D]`` are appended in place at ``cache_seqlens`` first and attention then covers
+    ``cache_seqlens + T`` tokens (with one query token ``causal`` changes nothing).  ``cache_seqlens`` itself
+    is not modified, as in flash-attn.  Returns ``out [B, 1, Hq, D]`` (and the natural-log LSE
+    ``[B, Hq, 1]`` fp32 with ``return_softmax_lse``).
+
+    Beyond flash-attn: ``cos_sin_cache`` + ``position_ids`` (the reference's rotary format) rotate q and k
+    on the way in, in the append launch; ``k_scale`` / ``v_scale`` select an fp8-e4m3 cache;
+    ``kv_lens_out`` receives ``cache_seqlens + T``.  ``num_splits`` 0 lets the library choose.
+    Not covered, and refused: more than one query token, flash-attn's own rotary arguments, left padding,
+    sliding windows and ALiBi.
+    """
+    if q.dim() != 4 or q.shape[1] != 1:
+        raise NotImplementedError("flash_attn_with_kvcache: this library covers the decode step (seqlen_q == 1)")
+    if rotary_cos is not None or rotary_sin is not None:
+        raise NotImplementedError("flash_attn_with_kvcache: pass cos_sin_cache= / position_ids= for rotary")
+    if cache_leftpad is not None or alibi_slopes is not None or tuple(window_size) != (-1, -1):
+        raise NotImplementedError("flash_attn_with_kvcache: cache_leftpad, alibi_slopes and window_size")
+    if cache_seqlens is None:
+        raise RuntimeError("flash_attn_with_kvcache: cache_seqlens is required")
+    bsz, _, q_heads, head_dim = q.shape
+    dev = q.device
+    if isinstance(cache_seqlens, int):
+        cache_seqlens = torch.full((bsz,), cache_seqlens, dtype=torch.int32, device=dev)
+    assert cache_seqlens.dtype == torch.int32 and cache_seqlens.numel() == bsz
+    if block_table is None:
+        if cache_batch_idx is not None:
+            block_table = cache_batch_idx.to(torch.int32).view(bsz, 1)
+        else:
+            assert k_cache.shape[0] >= bsz
+            block_table = _dense_block_table(dev, bsz)
+    elif cache_batch_idx is not None:
+        raise RuntimeError("flash_attn_with_kvcache: cache_batch_idx is not used with a paged cache")
+    scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
+
+    kv_lens = cache_seqlens
+    q_rot = q
+    if k is not None:
+        assert v is not None
+        if kv_lens_out is None:
+            kv_lens_out = torch.empty_like(cache_seqlens)
+        q_rot = rope_kv_append(k, v, k_cache, v_cache, block_table, cache_seqlens, kv_lens_out=kv_lens_out,
+                               k_scale=k_scale, v_scale=v_scale, cos_sin=cos_sin_cache, position_ids=position_ids,
+                               q=q if cos_sin_cache is not None else None, stream=stream)
+        if q_rot is None:
+            q_rot = q
+        kv_lens = kv_lens_out
+    elif cos_sin_cache is not None:
+        q_rot = rope_kv_append(None, None, None, None, None, None, cos_sin=cos_sin_cache, position_ids=position_ids,
+                               q=q, stream=stream)
+
+    out = torch.empty_like(q)
+    lse = torch.empty((bsz, q_heads), dtype=torch.float32, device=dev) if return_softmax_lse else None
+    _decode(q_rot.view(bsz, q_heads, head_dim) if q_rot.is_contiguous() else q_rot[:, 0], k_cache, v_cache, None,
+            kv_lens, block_table, scale, softcap, None, out.view(bsz, q_heads, head_dim),
+            num_splits if num_splits > 0 else -1, with_lse_column=False, lse_out=lse, k_scale=k_scale, v_scale=v_scale,
+            stream=stream, **decode_kw)
+    if return_softmax_lse:
+        return out, lse.view(bsz, q_heads, 1)
+    return out
