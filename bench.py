@@ -41,6 +41,8 @@ def parse_args():
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-write-side", action="store_true",
+                    help="skip the timing of the step before the decode (rotary + KV append)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
     ap.add_argument("--copy-ref", action="store_true",
@@ -50,6 +52,75 @@ def parse_args():
                     help="JSON file {\"traffic\": bytes per split-kernel launch} measured with the counter runs; "
                          "copied into roofline.traffic")
     return ap.parse_args()
+
+
+def _time_us(torch, fn, steps, warmup):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step):
+    """The step before the decode at this workload's shape: rotary of q and k plus the append of one token per
+    sequence (one launch), alone and followed by the decode step; and the same kernel at prefill size, where it is
+    an HBM-bound copy, priced against 8 TB/s with its algorithmic bytes (q, k, v read once; rotated q, K and V
+    written once; one cos/sin row per token)."""
+    B, Hq, D = wl.q.shape
+    _, P, Hkv, _ = wl.k_cache.shape
+    fp8 = wl.k_scale is not None
+    act = wl.q.dtype
+    cache_dtype = wl.k_cache.dtype
+    isz, csz = torch.empty(0, dtype=act).element_size(), wl.k_cache.element_size()
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.outer(torch.arange(8192, dtype=torch.float32), inv_freq)
+    cos_sin = torch.cat((ang.cos(), ang.sin()), dim=-1).to(dev)
+    scales = dict(k_scale=wl.k_scale, v_scale=wl.v_scale) if fp8 else {}
+
+    def setup(T):
+        pages = -(-(T + 1) // P)
+        kc = torch.zeros(B * pages, P, Hkv, D, dtype=cache_dtype, device=dev)
+        vc = torch.zeros_like(kc)
+        bt = torch.randperm(B * pages, device=dev).to(torch.int32).view(B, pages)
+        lens = torch.zeros(B, dtype=torch.int32, device=dev)
+        qkv = torch.randn(B, T, (Hq + 2 * Hkv) * D, device=dev).to(act)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        pos = torch.arange(T, device=dev).repeat(B, 1)
+        q4 = q.view(B, T, Hq, D)
+        q_out = torch.empty(B, T, Hq, D, dtype=act, device=dev)
+        lens_out = torch.empty_like(lens)
+
+        def run(_):
+            fd.rope_kv_append(k.view(B, T, Hkv, D), v.view(B, T, Hkv, D), kc, vc, bt, lens, kv_lens_out=lens_out,
+                              cos_sin=cos_sin, position_ids=pos, q=q4, q_out=q_out, **scales)
+        return run
+
+    one = setup(1)
+    t_append = _time_us(torch, one, steps, warmup)
+
+    def both(i):
+        one(i)
+        decode_step(i)
+    t_both = _time_us(torch, both, steps, warmup)
+
+    T = max(P, (4096 * 8 // B) // P * P)          # about 32k new tokens in total
+    big = setup(T)
+    t_big = _time_us(torch, big, max(5, steps // 5), 3)
+    tokens = B * T
+    nbytes = tokens * (2 * Hq * D * isz + 2 * Hkv * D * (isz + csz) + D * 4)
+    return {
+        "kernel": "fd_kv_append_kernel (rotary of q and k + paged append" + (" + fp8 quantisation)" if fp8 else ")"),
+        "decode_shape_us": round(t_append, 3), "append_plus_decode_step_us": round(t_both, 3),
+        "prefill_shape": {"new_tokens_per_seq": T, "us": round(t_big, 2), "algorithmic_bytes": nbytes,
+                          "achieved_gbps": round(nbytes / (t_big * 1e-6) / 1e9, 1),
+                          "frac_of_hbm_peak": round(nbytes / (t_big * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
+    }
 
 
 def main():
@@ -222,6 +293,9 @@ def main():
         result["mfma"] = {"useful_flop_per_step": wl_cpu.flops(), "issued_flop_per_step": int(issued),
                           "issued_tflops": round(issued / (split_us * 1e-6) / 1e12, 1),
                           "frac_of_dense_bf16_peak": round(issued / (split_us * 1e-6) / 2.5e15, 4)}
+
+    if not args.no_write_side:
+        result["write_side"] = measure_write_side(torch, fd, wl, dev, args.steps, args.warmup, step)
 
     if not args.no_cpu_baseline:
         import oracle  # the checker, timed as the CPU baseline only
