@@ -42,6 +42,14 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
   *shift = k;
 }
 
+// Shapes the MFMA split kernels are built for: head_dim 128 with a 16-bit or fp8-e4m3 cache, head_dim 256 with a
+// 16-bit cache; GQA group >= 4, and either <= 16 or a multiple of 16 (blocks of 16 query heads).
+bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
+  const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
+  const bool dim_ok = (head_dim == 128 && (kv16 || kv_dtype == FD_FP8_E4M3)) || (head_dim == 256 && kv16);
+  return dim_ok && group >= 4 && (group <= 16 || group % 16 == 0);
+}
+
 // Launch-shape policy, from sweeps on one MI355X (256 CUs): the kernels stream best with about
 // 1024 waves in flight, each walking a long token range (every wave pays a fixed prologue /
 // epilogue, and every split adds a partial for the combine), and with at least one workgroup per CU.
@@ -157,15 +165,14 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
   const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
-  const bool mfma_ok = D == 128 && G >= 4 && (G <= 16 || G % 16 == 0) && q16 &&
-                       (kv_fp8 || p->q_dtype == p->kv_dtype) &&
+  const bool mfma_ok = mfma_shape_ok(D, G, p->kv_dtype) && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
                        aligned16(q) && stride_q_bs % 8 == 0 && stride_q_h % 8 == 0;
   bool use_mfma = mfma_ok;
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs head_dim 128, group >= 4 (<= 16 or a multiple of 16), a 16-bit query with a "
-                "KV cache of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
+                "%s: MFMA path needs head_dim 128 (or 256 with a 16-bit cache), group >= 4 (<= 16 or a multiple of "
+                "16), a 16-bit query with a KV cache of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
@@ -174,7 +181,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (use_mfma) {
     a.hbsz = G < 16 ? G : 16;
     a.nhb = (G + 15) / 16;
-    tile = kv_fp8 ? 64 : 32;
+    tile = kv_fp8 ? 64 : (D == 256 ? 16 : 32);
   } else {
     a.hbsz = G >= 3 ? 4 : G;
     a.nhb = (G + a.hbsz - 1) / a.hbsz;
@@ -205,6 +212,8 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   int rc;
   if (use_mfma && kv_fp8) {
     rc = fd_launch_split_mfma_fp8((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
+  } else if (use_mfma && D == 256) {
+    rc = fd_launch_split_mfma_d256((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);
   } else if (use_mfma) {
     rc = fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);
   } else {
@@ -270,8 +279,7 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
       p->page_size <= 0 || p->max_pages_per_seq <= 0)
     return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0");
   const int G = p->q_heads / p->kv_heads;
-  const bool mfma = p->head_dim == 128 && G >= 4 && (G <= 16 || G % 16 == 0) && p->path != FD_PATH_VALU &&
-                    (p->kv_dtype == FD_FP8_E4M3 || p->kv_dtype == FD_F16 || p->kv_dtype == FD_BF16);
+  const bool mfma = mfma_shape_ok(p->head_dim, G, p->kv_dtype) && p->path != FD_PATH_VALU;
   const int64_t nhb = mfma ? (G + 15) / 16 : (G + (G >= 3 ? 4 : G) - 1) / (G >= 3 ? 4 : G);
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
