@@ -53,7 +53,8 @@ typedef enum fd_dtype {
 } fd_dtype;
 
 typedef enum fd_path {
-  FD_PATH_AUTO = 0,         /* MFMA when group >= 4, 16-bit/fp8 KV, head_dim 128   */
+  FD_PATH_AUTO = 0,         /* MFMA when group >= 4 and head_dim 128 (16-bit or fp8
+                               KV) or 256 (16-bit KV); else VALU                   */
   FD_PATH_VALU = 1,         /* force the VALU dot-product kernel                   */
   FD_PATH_MFMA = 2          /* force MFMA; FD_ERR_UNSUPPORTED if not applicable    */
 } fd_path;
@@ -202,8 +203,9 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
  * the partial workspace is internal, fewer and longer splits mean fewer workgroup
  * prologues and fewer partials for the combine.  Returns min(params->num_splits, the split
- * count that (1) reaches about 1024 waves with two waves per (KV head, split) and (2) keeps
- * every split of a full-length sequence at or below 4096 tokens), or a negative fd_status.
+ * count that (1) reaches about 1024 waves with two waves per (KV head, split) on the MFMA
+ * kernels, or about 2048 with four on the VALU kernel, and (2) keeps every split of a
+ * full-length sequence at or below 4096 tokens), or a negative fd_status.
  * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
  * params->num_splits splits with the reference's ranges.
  */

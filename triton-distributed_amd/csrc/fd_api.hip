@@ -50,19 +50,21 @@ bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
   return dim_ok && group >= 4 && (group <= 16 || group % 16 == 0);
 }
 
-// Launch-shape policy, from sweeps on one MI355X (256 CUs): the kernels stream best with about
-// 1024 waves in flight, each walking a long token range (every wave pays a fixed prologue /
-// epilogue, and every split adds a partial for the combine), and with at least one workgroup per CU.
+// Launch-shape policy, from sweeps on one MI355X (256 CUs): the MFMA kernels stream best with about
+// 1024 waves in flight (16 KB of loads each), the VALU kernel with about 2048 (8 KB each), each walking
+// a long token range (every wave pays a fixed prologue / epilogue, and every split adds a partial for
+// the combine), and with at least one workgroup per CU.
 constexpr int64_t kTargetWaves = 1024;
+constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = 4096;   // keeps a ragged batch balanceable by the dispatcher
 
 // Waves per (KV head, split) when the caller does not choose: the smallest power of two that reaches
 // kTargetWaves, never more waves than tiles a split can have.
-int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile) {
+int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, int64_t target) {
   int64_t tiles = (max_tokens_per_split + tile - 1) / tile;
   int w = 1;
-  while (w < 8 && head_splits * w < kTargetWaves && w * 2 <= tiles) w *= 2;
+  while (w < 8 && head_splits * w < target && w * 2 <= tiles) w *= 2;
   const char* env = getenv("FD_WAVES_PER_BLOCK");
   if (env) {
     int e = atoi(env);
@@ -190,7 +192,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
   const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
-  int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile);
+  int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile, use_mfma ? kTargetWaves : kTargetWavesValu);
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
@@ -283,8 +285,10 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   const int64_t nhb = mfma ? (G + 15) / 16 : (G + (G >= 3 ? 4 : G) - 1) / (G >= 3 ? 4 : G);
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
-  // (1) enough splits to reach the target wave count with two waves per head-split ...
-  int64_t s_fill = (kTargetWaves + 2 * groups - 1) / (2 * groups);
+  // (1) enough splits to reach the target wave count with two (MFMA) or four (VALU) waves per head-split ...
+  const int64_t per_split = mfma ? 2 * groups : 4 * groups;
+  const int64_t target = mfma ? kTargetWaves : kTargetWavesValu;
+  int64_t s_fill = (target + per_split - 1) / per_split;
   // (2) ... and enough that no split of a full-length sequence is longer than kMaxTokensPerSplit
   int64_t s_bal = (max_tokens + kMaxTokensPerSplit - 1) / kMaxTokensPerSplit;
   int64_t s = s_fill > s_bal ? s_fill : s_bal;
