@@ -167,6 +167,10 @@ FD_API int fd_combine(void* stream, const void* mid_o, const float* mid_lse, voi
  * fd_split_kv and fd_combine; out_split / lse_split are the partial workspace
  * (written, and readable by the caller afterwards).
  *
+ *  out_split NULL is allowed when params->num_splits == 1 and num_extra == 0: the single split's
+ *            normalised partial is the result, so the split kernel writes `out` (and lse_out,
+ *            or the LSE column in FD_COMBINE_SPLIT_LSE mode -- not both) directly and no
+ *            combine kernel is launched.
  *  tickets   NULL: two launches (split kernel, then combine kernel).
  *            Otherwise at least batch * q_heads int32, zero-initialised once by the
  *            caller and not shared by calls that may run concurrently: the combine is

@@ -446,3 +446,84 @@ def test_graph_capture_and_replay(fd, variant):
     ref, ref_lse = oracle_decode(wl.to("cpu"))
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
+
+
+# ---- single-split steps: the split kernel writes the output itself, no combine launch
+@pytest.mark.parametrize("kind", ["bf16", "fp16_d256", "fp8", "fp32_valu", "mha"])
+@pytest.mark.parametrize("variant", ["plain", "intra"])
+def test_large_batch_single_split_direct_output(fd, kind, variant):
+    import random
+    rng = random.Random(17)
+    B = 160
+    lens = [rng.randint(1, 300) for _ in range(B)]
+    lens[3] = 0
+    lens[77] = 0
+    Hq, Hkv, D, dtype, fp8 = {"bf16": (32, 8, 128, torch.bfloat16, False), "fp16_d256": (16, 4, 256, torch.float16, False),
+                              "fp8": (64, 8, 128, torch.bfloat16, True), "fp32_valu": (16, 8, 128, torch.float32, False),
+                              "mha": (8, 8, 128, torch.bfloat16, False)}[kind]
+    wl = fd.utils.make_paged_workload("direct", lens, Hq, Hkv, D, 16, dtype, 32, seed=23, fp8_kv=fp8)
+    # the plan for this shape is one split (enough (sequence, KV head) pairs to fill the chip)
+    from ctypes import byref
+    fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
+    g = wl.to(DEV)
+    p = fk._make_params(g.q, g.k_cache, g.block_table, 32, 0.0, 0, 0, g.k_scale, g.v_scale, "auto", 0)
+    assert fd.load_library().fd_plan_splits(byref(p), B) == 1
+    out, lse = run_decode(fd, wl, variant=variant) if variant == "plain" else (None, None)
+    ref, ref_lse = oracle_decode(wl)
+    atol = 2e-4 if dtype == torch.float32 else 2e-2
+    if variant == "plain":
+        assert_out_close(out, ref, atol=atol)
+        assert_lse_close(lse, ref_lse, rtol=1e-5 if dtype == torch.float32 else 1e-3)
+        # without an LSE request nothing is written beyond the [B, Hq, D] rows
+        canary = torch.full((B, Hq, D + 8), 7.0, dtype=g.q.dtype, device=DEV)
+        kw = dict(k_scale=g.k_scale, v_scale=g.v_scale) if fp8 else {}
+        fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
+                                output_combine=canary[..., :D], kv_split=32, **kw)
+        torch.cuda.synchronize()
+        assert_out_close(canary[..., :D].cpu(), ref, atol=atol)
+        assert (canary[..., D:] == 7.0).all()
+    else:
+        kw = dict(k_scale=g.k_scale, v_scale=g.v_scale) if fp8 else {}
+        res = fd.gqa_fwd_batch_decode_intra_rank(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
+                                                 kv_split=32, **kw)
+        torch.cuda.synchronize()
+        assert res.shape == (B, Hq, D + 1)
+        assert_out_close(res[..., :D].cpu(), ref, atol=atol)
+        # the LSE column has the output's dtype
+        assert_lse_close(res[..., D].float().cpu(), ref_lse, rtol=1e-5 if dtype == torch.float32 else 1e-2)
+    # two launches on the same inputs (exactly one split into a caller buffer, then the combine): same bits
+    if not fp8:
+        two = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
+                                      kv_split=1, output_split=torch.empty(B, Hq, 1, D + 1, dtype=torch.float32,
+                                                                           device=DEV))
+        one = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
+                                      kv_split=32)
+        torch.cuda.synchronize()
+        assert torch.equal(one.cpu().view(torch.uint8), two.cpu().view(torch.uint8))
+
+
+def test_direct_output_c_abi_rules(fd):
+    from ctypes import byref
+    lib = fd.load_library()
+    fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
+    wl = fd.utils.make_paged_workload("direct_abi", [40, 9], 8, 2, 128, 16, torch.bfloat16, 32, seed=5).to(DEV)
+    out = torch.empty(2, 8, 128, dtype=torch.bfloat16, device=DEV)
+    lse = torch.empty(2, 8, dtype=torch.float32, device=DEV)
+
+    def call(S, mode, lse_ptr, n_extra=0):
+        p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S, 0.0, fd._lib.FD_F32, fd._lib.FD_BF16, None, None, "auto", 0)
+        return lib.fd_decode(None, wl.q.data_ptr(), wl.k_cache.data_ptr(), wl.v_cache.data_ptr(), None, None,
+                             out.data_ptr(), lse_ptr, float(wl.scale), wl.block_table.data_ptr(), wl.kv_lens.data_ptr(), 2,
+                             wl.q.stride(0), wl.q.stride(1), wl.k_cache.stride(-3), wl.k_cache.stride(-2),
+                             wl.v_cache.stride(-3), wl.v_cache.stride(-2), 0, 0, 0, wl.block_table.stride(0),
+                             out.stride(0), out.stride(1), None, mode, out.data_ptr() if n_extra else None,
+                             lse.data_ptr() if n_extra else None, n_extra, None, byref(p))
+
+    assert call(2, fd._lib.FD_COMBINE_SPLIT, lse.data_ptr()) < 0 and b"out_split may be NULL only" in lib.fd_last_error()
+    assert call(1, fd._lib.FD_COMBINE_SPLIT, lse.data_ptr(), n_extra=1) < 0
+    assert call(1, fd._lib.FD_COMBINE_SPLIT_LSE, lse.data_ptr()) < 0 and b"not both" in lib.fd_last_error()
+    assert call(1, fd._lib.FD_COMBINE_SPLIT, lse.data_ptr()) == 0
+    torch.cuda.synchronize()
+    ref, ref_lse = oracle_decode(wl.to("cpu"))
+    assert_out_close(out.cpu(), ref)
+    assert_lse_close(lse.cpu(), ref_lse)

@@ -111,7 +111,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
                const int32_t* kv_lens, int32_t batch, int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok,
                int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
                int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p,
-               const FusedTail* tail, bool* fused) {
+               const FusedTail* tail, bool* fused, bool no_lse = false) {
   if (fused) *fused = false;
   if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (!q || !k_cache || !v_cache || !out_split || !block_table || !kv_lens)
@@ -155,7 +155,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   a.k_scale = p->k_scale; a.v_scale = p->v_scale;
   a.sq_b = stride_q_bs; a.sq_h = stride_q_h; a.sk_t = stride_k_tok; a.sk_h = stride_k_h;
   a.sv_t = stride_v_tok; a.sv_h = stride_v_h; a.so_b = stride_o_bs; a.so_h = stride_o_h; a.so_s = stride_o_split;
-  a.sbt = stride_table_bs;
+  a.sbt = stride_table_bs; a.no_lse = no_lse ? 1 : 0;
   a.sm_scale = sm_scale; a.soft_cap = p->soft_cap > 0.f ? p->soft_cap : 0.f;
   a.batch = batch; a.Hq = p->q_heads; a.Hkv = p->kv_heads; a.G = G; a.S = p->num_splits; a.P = p->page_size;
   div_magic((uint32_t)p->page_size, &a.div_magic, &a.div_shift);
@@ -261,6 +261,21 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
     return fail(FD_ERR_INVALID_ARG, "fd_decode: num_extra %d needs extra_out and extra_lse", num_extra);
   if (p && (!dtype_size(p->out_dtype) || p->out_dtype == FD_FP8_E4M3))
     return fail(FD_ERR_UNSUPPORTED, "fd_decode: out_dtype %d", p->out_dtype);
+  if (!out_split) {
+    // One split and nothing else to merge: its normalised partial IS the result.  The split kernel writes
+    // it (and the LSE) in the output's place and dtype; no combine launch.
+    if (!p) return fail(FD_ERR_INVALID_ARG, "fd_decode: params is NULL");
+    if (p->num_splits != 1 || num_extra != 0)
+      return fail(FD_ERR_INVALID_ARG, "fd_decode: out_split may be NULL only with num_splits == 1 and no extra partials");
+    if (combine_mode == FD_COMBINE_SPLIT_LSE && lse_out)
+      return fail(FD_ERR_INVALID_ARG, "fd_decode: without out_split the LSE goes to lse_out or to the output column, not both");
+    fd_params direct = *p;
+    direct.mid_dtype = p->out_dtype;
+    return split_impl("fd_decode", stream, q, k_cache, v_cache, out, lse_out, sm_scale, block_table, kv_lens, batch,
+                      stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_obs, stride_oh,
+                      0, stride_table_bs, seq_order, &direct, nullptr, nullptr,
+                      combine_mode == FD_COMBINE_SPLIT && !lse_out);
+  }
   FusedTail tail;
   tail.tickets = tickets; tail.out = out; tail.lse_out = lse_out; tail.extra_out = extra_out;
   tail.extra_lse = extra_lse; tail.stride_obs = stride_obs; tail.stride_oh = stride_oh; tail.num_extra = num_extra;

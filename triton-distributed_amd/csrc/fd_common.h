@@ -43,6 +43,7 @@ struct SplitArgs {
   int32_t hbsz;     // query heads per head block
   int32_t hpw;      // adjacent KV heads per workgroup (one wave each; x token sub-ranges = waves)
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
+  int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
@@ -268,7 +269,7 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
       } else {
         for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
       }
-      if (d == 0) {
+      if (d == 0 && !a.no_lse) {
         if (a.lse) {
           a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
         } else {

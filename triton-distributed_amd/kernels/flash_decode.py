@@ -147,7 +147,12 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             num_splits = planned
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
-        if (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
+        direct = (num_splits == 1 and extra_partials is None and not fuse_combine
+                  and not (with_lse_column and lse_out is not None))
+        if direct:
+            # a single split: the split kernel writes the output itself, no partials and no combine launch
+            hold = None
+        elif (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
                 and workspace.is_contiguous() and workspace.numel() >= n_o + n_l):
             # a float32 workspace that is large enough holds the partials: no allocation in the call
             hold = workspace
@@ -155,8 +160,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             hold = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
             if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
                 hold.record_stream(stream)
-        mid_ptr = hold.data_ptr()
-        lse_split_ptr = mid_ptr + 4 * n_o
+        mid_ptr = hold.data_ptr() if hold is not None else None
+        lse_split_ptr = mid_ptr + 4 * n_o if hold is not None else None
         mid_dtype = FD_F32
         so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
     else:
