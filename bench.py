@@ -67,7 +67,7 @@ def _time_us(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) * 1e3 / steps
 
 
-def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step):
+def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step, pools, kv_split):
     """The step before the decode at this workload's shape: rotary of q and k plus the append of one token per
     sequence (one launch), alone and followed by the decode step; and the same kernel at prefill size, where it is
     an HBM-bound copy, priced against 8 TB/s with its algorithmic bytes (q, k, v read once; rotated q, K and V
@@ -109,6 +109,20 @@ def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step):
         decode_step(i)
     t_both = _time_us(torch, both, steps, warmup)
 
+    # the drop-in call of the reference's attention block on this workload's own pools: rotary + append (which also
+    # ranks the sequences for the decode's issue order when the batch is large enough) + split-KV decode + combine
+    qkv1 = torch.randn(B, 1, (Hq + 2 * Hkv) * D, device=dev).to(act)
+    q1, k1, v1 = [t.view(B, 1, -1, D) for t in qkv1.split([Hq * D, Hkv * D, Hkv * D], dim=-1)]
+    pos1 = wl.kv_lens[:, None].long().clamp(max=cos_sin.shape[0] - 1)
+    grown = torch.empty_like(wl.kv_lens)
+
+    def fused(i):
+        k, v = pools[i % len(pools)]
+        fd.flash_attn_with_kvcache(q1, k, v, k=k1, v=v1, cache_seqlens=wl.kv_lens, block_table=wl.block_table,
+                                   causal=True, softcap=wl.soft_cap, num_splits=kv_split, cos_sin_cache=cos_sin,
+                                   position_ids=pos1, kv_lens_out=grown, **scales)
+    t_fused = _time_us(torch, fused, steps, warmup)
+
     T = max(P, (4096 * 8 // B) // P * P)          # about 32k new tokens in total
     big = setup(T)
     t_big = _time_us(torch, big, max(5, steps // 5), 3)
@@ -117,6 +131,7 @@ def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step):
     return {
         "kernel": "fd_kv_append_kernel (rotary of q and k + paged append" + (" + fp8 quantisation)" if fp8 else ")"),
         "decode_shape_us": round(t_append, 3), "append_plus_decode_step_us": round(t_both, 3),
+        "flash_attn_with_kvcache_us": round(t_fused, 3),
         "prefill_shape": {"new_tokens_per_seq": T, "us": round(t_big, 2), "algorithmic_bytes": nbytes,
                           "achieved_gbps": round(nbytes / (t_big * 1e-6) / 1e9, 1),
                           "frac_of_hbm_peak": round(nbytes / (t_big * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
@@ -295,7 +310,7 @@ def main():
                           "frac_of_dense_bf16_peak": round(issued / (split_us * 1e-6) / 2.5e15, 4)}
 
     if not args.no_write_side:
-        result["write_side"] = measure_write_side(torch, fd, wl, dev, args.steps, args.warmup, step)
+        result["write_side"] = measure_write_side(torch, fd, wl, dev, args.steps, args.warmup, step, pools, S)
 
     if not args.no_cpu_baseline:
         import oracle  # the checker, timed as the CPU baseline only

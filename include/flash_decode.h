@@ -253,11 +253,14 @@ typedef struct fd_rope {
  *                contiguous, 16-byte aligned rows.  Both NULL: only rope->q is processed.
  *  kv_lens       [batch] tokens already in the cache (not modified)
  *  kv_lens_out   NULL, or [batch] (not kv_lens itself): min(kv_lens[b] + new_tokens, capacity)
+ *  seq_order_out NULL, or [batch] int32 (batch <= 4096): what fd_schedule would return for
+ *                kv_lens_out -- the issue order for the decode that follows, computed by a few
+ *                trailing workgroups of this launch instead of a launch of its own
  *  A token whose position is at or beyond max_pages_per_seq * page_size is not written.
  */
 FD_API int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                  const int32_t* block_table, const int32_t* kv_lens, int32_t* kv_lens_out,
-                 int32_t batch, int32_t new_tokens,
+                 int32_t* seq_order_out, int32_t batch, int32_t new_tokens,
                  int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
                  int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h,
                  int64_t stride_k_tok, int64_t stride_k_h,

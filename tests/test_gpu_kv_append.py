@@ -184,7 +184,7 @@ def test_error_paths(fd):
         p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_pages, p.max_pages_per_seq = 1, Hkv, D, P, 8, 2
         p.q_dtype, p.kv_dtype = fd._lib.FD_BF16, fd._lib.FD_FP8_E4M3
         fd._lib.check(lib.fd_kv_append(None, k.data_ptr(), k.data_ptr(), kc.data_ptr(), kc.data_ptr(), bt.data_ptr(),
-                                       lens.data_ptr(), None, B, T, *k.stride()[:3], *k.stride()[:3], kc.stride(1),
+                                       lens.data_ptr(), None, None, B, T, *k.stride()[:3], *k.stride()[:3], kc.stride(1),
                                        kc.stride(2), kc.stride(1), kc.stride(2), bt.stride(0), None, byref(p)))
     with pytest.raises(RuntimeError, match="16-byte aligned"):
         kk = torch.zeros(B, T, Hkv, D + 1, dtype=torch.bfloat16, device=DEV)[..., 1:]
@@ -274,3 +274,55 @@ def test_flash_attn_with_kvcache_decode_step(fd, layout, fp8, rope):
     assert torch.equal(vc_g.cpu().view(torch.uint8), ref_vc.view(torch.uint8))
     assert_out_close(out[:, 0], ref)
     assert_lse_close(lse[..., 0], ref_lse)
+
+
+def test_append_also_ranks_sequences(fd):
+    """seq_order_out of the append launch == the stand-alone scheduler on the grown lengths (ties by index,
+    lengths capped at the table's capacity), and flash_attn_with_kvcache uses it for batches of 16 and more."""
+    gen = torch.Generator().manual_seed(4)
+    B, Hq, Hkv, D, P = 300, 8, 2, 128, 16
+    lens = torch.randint(0, 48, (B,), generator=gen, dtype=torch.int32)
+    lens[5] = lens[9] = lens[200] = 47          # ties, and 47 + 2 new tokens exceeds the capacity of 48
+    bt = torch.randperm(B * 3, generator=gen).to(torch.int32).view(B, 3).to(DEV)
+    k = torch.randn(B, 2, Hkv, D, generator=gen).to(torch.bfloat16).to(DEV)
+    kc = torch.zeros(B * 3, P, Hkv, D, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    grown = torch.empty(B, dtype=torch.int32, device=DEV)
+    order = torch.full((B,), -1, dtype=torch.int32, device=DEV)
+    fd.paged_kv_append(k, k, kc, vc, bt, lens.to(DEV), kv_lens_out=grown, seq_order_out=order)
+    want = fd.schedule_sequences(grown)
+    torch.cuda.synchronize()
+    assert torch.equal(grown.cpu(), (lens + 2).clamp(max=48))
+    assert torch.equal(order.cpu(), want.cpu())
+    ref = sorted(range(B), key=lambda i: (-int(grown[i]), i))
+    assert order.cpu().tolist() == ref
+
+    # the decode-step call: ragged batch of 24 sequences, oracle on the CPU
+    B = 24
+    lens = torch.randint(0, 600, (B,), generator=gen, dtype=torch.int32)
+    pages = 40
+    bt = torch.randperm(B * pages, generator=gen).to(torch.int32).view(B, pages)
+    kc = torch.randn(B * pages, P, Hkv, D, generator=gen).to(torch.bfloat16)
+    vc = torch.randn(B * pages, P, Hkv, D, generator=gen).to(torch.bfloat16)
+    q = torch.randn(B, 1, Hq, D, generator=gen).to(torch.bfloat16)
+    k = torch.randn(B, 1, Hkv, D, generator=gen).to(torch.bfloat16)
+    v = torch.randn(B, 1, Hkv, D, generator=gen).to(torch.bfloat16)
+    ref_k, ref_v = kc.clone(), vc.clone()
+    new_lens = oracle.ref_kv_append(k, v, ref_k, ref_v, bt, lens)
+    ref, _ = oracle.ref_paged_attn_lse(q[:, 0].float(), ref_k.float(), ref_v.float(), new_lens.tolist(), bt, D ** -0.5)
+    seen = {}
+    real = fd.kernels.kv_append._decode
+
+    def spy(*a, **kw):
+        seen["order"] = kw.get("seq_order")
+        return real(*a, **kw)
+    fd.kernels.kv_append._decode = spy
+    try:
+        out = fd.flash_attn_with_kvcache(q.to(DEV), kc.to(DEV), vc.to(DEV), k=k.to(DEV), v=v.to(DEV),
+                                         cache_seqlens=lens.to(DEV), block_table=bt.to(DEV), causal=True)
+    finally:
+        fd.kernels.kv_append._decode = real
+    torch.cuda.synchronize()
+    assert seen["order"] is not None
+    assert seen["order"].cpu().tolist() == sorted(range(B), key=lambda i: (-int(new_lens[i]), i))
+    assert_out_close(out[:, 0], ref)

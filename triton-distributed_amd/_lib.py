@@ -99,7 +99,7 @@ def load_library(path: str = None) -> ctypes.CDLL:
     lib.fd_plan_splits.argtypes = [POINTER(FdParams), c_int32]
     lib.fd_kv_append.restype = c_int32
     lib.fd_kv_append.argtypes = [
-        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
         i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, POINTER(FdRope), POINTER(FdParams)]
     lib.fd_schedule.restype = c_int32
     lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]

@@ -358,8 +358,8 @@ int fd_combine(void* stream, const void* mid_o, const float* mid_lse, void* out,
 }
 
 int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
-                 const int32_t* block_table, const int32_t* kv_lens, int32_t* kv_lens_out, int32_t batch,
-                 int32_t new_tokens, int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
+                 const int32_t* block_table, const int32_t* kv_lens, int32_t* kv_lens_out, int32_t* seq_order_out,
+                 int32_t batch, int32_t new_tokens, int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
                  int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h, int64_t stride_k_tok,
                  int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_table_bs,
                  const fd_rope* rope, const fd_params* p) {
@@ -369,6 +369,9 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
   if (batch == 0 || new_tokens == 0) return FD_OK;
   const bool append = k_new || v_new;
   const bool with_q = rope && rope->q;
+  if (seq_order_out && !append) return fail(FD_ERR_INVALID_ARG, "%s: seq_order_out needs k_new / v_new and kv_lens", fn);
+  if (seq_order_out && batch > 4096)
+    return fail(FD_ERR_TOO_LARGE, "%s: seq_order_out with batch %d > 4096 (use fd_schedule)", fn, batch);
   if (!append && !with_q) return fail(FD_ERR_INVALID_ARG, "%s: nothing to do (no k_new / v_new and no rope->q)", fn);
   const int D = p->head_dim;
   if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "%s: head_dim %d (64/128/256)", fn, D);
@@ -407,7 +410,7 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
       return fail(FD_ERR_ALIGNMENT, "%s: k_new / v_new rows must be 16-byte aligned (pointer and strides)", fn);
     if (stride_k_tok <= 0 || stride_v_tok <= 0) return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
     a.k_new = k_new; a.v_new = v_new; a.k_cache = k_cache; a.v_cache = v_cache;
-    a.bt = block_table; a.kv_lens = kv_lens; a.kv_lens_out = kv_lens_out;
+    a.bt = block_table; a.kv_lens = kv_lens; a.kv_lens_out = kv_lens_out; a.seq_order = seq_order_out;
     a.k_scale = p->k_scale; a.v_scale = p->v_scale;
     a.skn_b = stride_kn_b; a.skn_t = stride_kn_t; a.skn_h = stride_kn_h;
     a.svn_b = stride_vn_b; a.svn_t = stride_vn_t; a.svn_h = stride_vn_h;

@@ -80,6 +80,8 @@ struct AppendArgs {
   const int32_t* bt;
   const int32_t* kv_lens;
   int32_t* kv_lens_out;  // nullptr or [batch]
+  int32_t* seq_order;    // nullptr or [batch]: sequences ranked by grown length, longest first
+  int32_t data_blocks;   // workgroups that move data; the ones after them compute seq_order
   const float* k_scale;
   const float* v_scale;
   int64_t skn_b, skn_t, skn_h, svn_b, svn_t, svn_h, sk_t, sk_h, sv_t, sv_h, sbt;

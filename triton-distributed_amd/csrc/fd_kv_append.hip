@@ -98,6 +98,26 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
   const int hq = a.q ? a.Hq : 0;
   const int hkv = a.k_new ? a.Hkv : 0;
   const int heads = hq + 2 * hkv;               // rows per (sequence, token): K heads, V heads, Q heads
+  if ((int)blockIdx.x >= a.data_blocks) {
+    // Trailing workgroups: issue order for the decode that follows (same ranking as the stand-alone
+    // scheduler: grown length descending, ties by index), so that it costs no launch of its own.
+    const int i = ((int)blockIdx.x - a.data_blocks) * blockDim.x + threadIdx.x;
+    if (i >= a.batch) return;
+    const int64_t cap = (int64_t)a.max_pages * a.P;
+    auto grown = [&](int b) {
+      int64_t len = a.kv_lens[b];
+      len = (len < 0 ? 0 : len) + a.T;
+      return len > cap ? cap : len;
+    };
+    const int64_t mine = grown(i);
+    int rank = 0;
+    for (int j = 0; j < a.batch; ++j) {
+      const int64_t other = grown(j);
+      rank += (other > mine) || (other == mine && j < i);
+    }
+    a.seq_order[rank] = i;
+    return;
+  }
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t row = g / cpr;
   if (row >= (int64_t)a.batch * a.T * heads) return;
@@ -179,12 +199,15 @@ int launch_src(hipStream_t stream, const AppendArgs& a, int kv_dtype, dim3 grid)
 
 }  // namespace
 
-int fd_launch_kv_append(hipStream_t stream, const AppendArgs& a, int src_dtype, int kv_dtype) {
+int fd_launch_kv_append(hipStream_t stream, const AppendArgs& args, int src_dtype, int kv_dtype) {
+  AppendArgs a = args;
   const int heads = (a.q ? a.Hq : 0) + (a.k_new ? 2 * a.Hkv : 0);
   const int64_t threads = (int64_t)a.batch * a.T * heads * (a.D >> 4);
   if (threads == 0) return FD_OK;
-  const int64_t blocks = (threads + 255) / 256;
-  if (blocks > 0x7fffffffLL) return FD_ERR_TOO_LARGE;
+  int64_t blocks = (threads + 255) / 256;
+  if (blocks > 0x7fff0000LL) return FD_ERR_TOO_LARGE;
+  a.data_blocks = (int32_t)blocks;
+  if (a.seq_order) blocks += (a.batch + 255) / 256;
   const dim3 grid((unsigned)blocks);
   switch (src_dtype) {
     case FD_F32: return launch_src<float>(stream, a, kv_dtype, grid);

@@ -41,6 +41,7 @@ def _rope_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdRope:
 def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                    v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                    kv_lens: Optional[torch.Tensor], *, kv_lens_out: Optional[torch.Tensor] = None,
+                   seq_order_out: Optional[torch.Tensor] = None,
                    k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
                    cos_sin: Optional[torch.Tensor] = None, position_ids: Optional[torch.Tensor] = None,
                    q: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None, stream=None):
@@ -50,14 +51,17 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
     is stored and ``q`` ``[B, T, Hq, D]`` (if given) is rotated into ``q_out`` (default: a new tensor; may be
     ``q``) in the same launch.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
     ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out`` (int32 ``[B]``, not ``kv_lens``) receives
-    the grown lengths.  Returns ``q_out`` (or ``None`` without ``q``).
+    the grown lengths; ``seq_order_out`` (int32 ``[B]``, ``B <= 4096``) the longest-first issue order for the
+    decode that follows (what ``schedule_sequences`` would compute, without a launch of its own).  Returns
+    ``q_out`` (or ``None`` without ``q``).
     """
     lib = load_library()
     append = k_new is not None
     src = k_new if append else q
     if src is None:
         raise RuntimeError("rope_kv_append: neither k_new nor q given")
-    _require_cuda(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out, cos_sin, position_ids, q, q_out)
+    _require_cuda(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out, seq_order_out, cos_sin,
+                  position_ids, q, q_out)
     bsz, seq, _, head_dim = src.shape
     p = FdParams()
     p.head_dim = head_dim
@@ -80,6 +84,8 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
             raise RuntimeError("k_scale and v_scale must be given together")
         if kv_lens_out is not None:
             assert kv_lens_out.dtype == torch.int32 and kv_lens_out.is_contiguous() and kv_lens_out.numel() == bsz
+        if seq_order_out is not None:
+            assert seq_order_out.dtype == torch.int32 and seq_order_out.is_contiguous() and seq_order_out.numel() == bsz
         p.page_size = page_size
         p.num_pages = k_cache.shape[0]
         p.max_pages_per_seq = block_table.shape[1]
@@ -104,16 +110,16 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
         raise RuntimeError("rope_kv_append: q is only processed together with cos_sin / position_ids")
     check(lib.fd_kv_append(
         stream_handle(stream, src.device.index), ptr(k_new), ptr(v_new), ptr(k_cache), ptr(v_cache), ptr(block_table),
-        ptr(kv_lens), ptr(kv_lens_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
+        ptr(kv_lens), ptr(kv_lens_out), ptr(seq_order_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
         byref(rope) if rope is not None else None, byref(p)))
     return q_out if q is not None else None
 
 
-def paged_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, *, kv_lens_out=None, k_scale=None,
-                    v_scale=None, stream=None):
+def paged_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, *, kv_lens_out=None, seq_order_out=None,
+                    k_scale=None, v_scale=None, stream=None):
     """``rope_kv_append`` without the rotation: the plain cache update (models/kv_cache.py:43-50 for a paged pool)."""
-    rope_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out=kv_lens_out, k_scale=k_scale,
-                   v_scale=v_scale, stream=stream)
+    rope_kv_append(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out=kv_lens_out,
+                   seq_order_out=seq_order_out, k_scale=k_scale, v_scale=v_scale, stream=stream)
 
 
 def apply_rotary_pos_emb(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: torch.Tensor) -> torch.Tensor:
@@ -126,6 +132,9 @@ def apply_rotary_pos_emb(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: t
 
 
 _ARANGE = {}
+# Batches for which flash_attn_with_kvcache lets the append launch rank the sequences: below, every sequence's
+# workgroups start at once anyway; above, one thread per sequence ranking against all others gets long.
+SCHEDULE_MIN_BATCH, SCHEDULE_MAX_BATCH = 16, 1024
 
 
 def _dense_block_table(device, n):
@@ -187,8 +196,11 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
         assert v is not None
         if kv_lens_out is None:
             kv_lens_out = torch.empty_like(cache_seqlens)
+        if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw:
+            # the append launch also ranks the sequences (longest first) for the decode's issue order
+            decode_kw["seq_order"] = torch.empty_like(cache_seqlens)
         q_rot = rope_kv_append(k, v, k_cache, v_cache, block_table, cache_seqlens, kv_lens_out=kv_lens_out,
-                               k_scale=k_scale, v_scale=v_scale, cos_sin=cos_sin_cache, position_ids=position_ids,
+                               seq_order_out=decode_kw.get("seq_order"), k_scale=k_scale, v_scale=v_scale, cos_sin=cos_sin_cache, position_ids=position_ids,
                                q=q if cos_sin_cache is not None else None, stream=stream)
         if q_rot is None:
             q_rot = q
