@@ -216,26 +216,34 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
 FD_API int fd_plan_splits(const fd_params* params, int32_t batch);
 
 /*
- * Rotary position embedding applied on the way into the cache, as the reference's
- * apply_rotary_pos_emb does right before its cache update
- * (python/triton_dist/layers/amd/tp_attn.py:72-125 kernel, :128-160 launch, :232-241 and
- * :263-264 call sites): out[i] = x[i]*cos[i] - x[i+D/2]*sin[i],
- * out[i+D/2] = x[i+D/2]*cos[i] + x[i]*sin[i] for i < D/2, in fp32, each product and sum
- * rounded separately, the result rounded to the activation dtype.
+ * What the reference's attention block does to q and k between the QKV projection and the
+ * cache update (python/triton_dist/layers/amd/tp_attn.py:252-264), applied on the way in:
+ *
+ *  1. optional per-head RMS norm over head_dim (`layer_norm`, tp_attn.py:52-59, 252-258):
+ *     y = x * rsqrt(mean(x^2) + eps) * w in fp32, rounded to the activation dtype;
+ *  2. optional rotary position embedding (apply_rotary_pos_emb, tp_attn.py:72-125 kernel,
+ *     :128-160 launch, :232-241 and :263-264 call sites): out[i] = x[i]*cos[i] - x[i+D/2]*sin[i],
+ *     out[i+D/2] = x[i+D/2]*cos[i] + x[i]*sin[i] for i < D/2, in fp32, each product and sum
+ *     rounded separately, the result rounded to the activation dtype.
+ *
+ * K rows get both before they are stored; q rows (if given) get both into q_out.
  */
-typedef struct fd_rope {
-  const float* cos_sin;       /* [max_positions, D] fp32: D/2 cosines then D/2 sines per row
-                                 (tp_attn.py:62-69), 16-byte aligned rows                  */
+typedef struct fd_qk_prep {
+  const float* cos_sin;       /* NULL (no rotation), or [max_positions, D] fp32: D/2 cosines
+                                 then D/2 sines per row (tp_attn.py:62-69), 16-byte aligned  */
   int64_t stride_cos_sin;     /* row stride in elements                                    */
   const void* position_ids;   /* [batch, new_tokens]                                       */
   int32_t position_dtype;     /* 0: int32, 1: int64                                        */
   int32_t max_positions;      /* positions are clamped into [0, max_positions)             */
   int64_t stride_pos_b, stride_pos_t;
   const void* q;              /* NULL, or [batch, new_tokens, Hq, D] in params->q_dtype     */
-  void* q_out;                /* rotated q, same dtype; may be q itself                    */
+  void* q_out;                /* processed q, same dtype; may be q itself                  */
   int64_t stride_q_b, stride_q_t, stride_q_h;
   int64_t stride_qo_b, stride_qo_t, stride_qo_h;
-} fd_rope;
+  const void* q_norm_weight;  /* NULL (no norm of q), or [D] in params->q_dtype, 16-byte aligned */
+  const void* k_norm_weight;  /* NULL (no norm of k), or [D] in params->q_dtype, 16-byte aligned */
+  float q_norm_eps, k_norm_eps;
+} fd_qk_prep;
 
 /*
  * The step before the decode: appends `new_tokens` tokens of K and V per sequence to the
@@ -246,11 +254,11 @@ typedef struct fd_rope {
  * reads (python/triton_dist/test/nvidia/test_decode_attn.py:150-156); the reference itself
  * only has a dense cache whose update is a slice assignment
  * (python/triton_dist/models/kv_cache.py:43-50, called at layers/amd/tp_attn.py:265), which
- * is this layout with one page per sequence.  With `rope`, K is rotated before it is stored
- * and, if rope->q is given, Q is rotated in the same launch.
+ * is this layout with one page per sequence.  With `prep`, K is normalised and / or rotated
+ * before it is stored and, if prep->q is given, so is Q in the same launch.
  *
  *  k_new, v_new  [batch, new_tokens, Hkv, D], element strides stride_*n_b / _t / _h, last dim
- *                contiguous, 16-byte aligned rows.  Both NULL: only rope->q is processed.
+ *                contiguous, 16-byte aligned rows.  Both NULL: only prep->q is processed.
  *  kv_lens       [batch] tokens already in the cache (not modified)
  *  kv_lens_out   NULL, or [batch] (not kv_lens itself): min(kv_lens[b] + new_tokens, capacity)
  *  seq_order_out NULL, or [batch] int32 (batch <= 4096): what fd_schedule would return for
@@ -265,7 +273,7 @@ FD_API int fd_kv_append(void* stream, const void* k_new, const void* v_new, void
                  int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h,
                  int64_t stride_k_tok, int64_t stride_k_h,
                  int64_t stride_v_tok, int64_t stride_v_h,
-                 int64_t stride_table_bs, const fd_rope* rope, const fd_params* params);
+                 int64_t stride_table_bs, const fd_qk_prep* prep, const fd_params* params);
 
 /* Message for the last non-zero status returned on this thread ("" if none). */
 FD_API const char* fd_last_error(void);

@@ -16,6 +16,7 @@ from .ref_decode import (  # noqa: F401
 from .ref_kv_append import (  # noqa: F401
     ref_set_cos_sin_cache,
     ref_rope,
+    ref_rms_norm,
     ref_quantize_fp8,
     brute_force_fp8,
     ref_kv_append,

@@ -20,7 +20,12 @@ update here is "token n of sequence b lives at page ``block_table[b, n // P]``, 
 ``n % P``" -- the inverse of that gather.  fp8 caches store
 ``clamp(x / scale[kv head], +-448)`` rounded to e4m3fn (nearest even).
 
-Pinning status (tests/test_oracle_pinning.py): the rotation by complex multiplication in
+``ref_rms_norm`` restates the per-head RMS norm the block applies to q and k before the rotation
+(``tp_attn.py:52-59, 252-258``); it is evaluated in float64, so a float32 implementation agrees with it
+to rounding of the activation dtype, not bit for bit.
+
+Pinning status (tests/test_oracle_pinning.py): the norm by ``torch.nn.functional.rms_norm`` (fp32, CPU), by
+scale invariance at eps = 0 and by the constant-row closed form; the rotation by complex multiplication in
 float64, by norm preservation, by position 0 being the identity and by additivity of
 angles; the table by its definition at hand-computed points; the append by the round trip
 through ``ref_decode._gather_kv`` (append token by token, gather, compare with the source
@@ -59,6 +64,14 @@ def ref_rope(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: torch.Tensor)
     o2 = (x2 * cos).astype(np.float32) + (x1 * sin).astype(np.float32)
     out = np.concatenate([o1, o2], axis=-1).astype(np.float32)
     return torch.from_numpy(out).to(x.dtype)
+
+
+def ref_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Per-row RMS norm over the last dimension, ``x * rsqrt(mean(x^2) + eps) * w`` (tp_attn.py:52-59: torch's
+    ``rms_norm`` on the rows of ``[.., heads, head_dim]``), evaluated in float64 and rounded once to x's dtype."""
+    xd = x.to(torch.float64)
+    rstd = torch.rsqrt(xd.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (xd * rstd * weight.to(torch.float64)).to(x.dtype)
 
 
 def ref_quantize_fp8(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:

@@ -326,3 +326,63 @@ def test_append_also_ranks_sequences(fd):
     assert seen["order"] is not None
     assert seen["order"].cpu().tolist() == sorted(range(B), key=lambda i: (-int(new_lens[i]), i))
     assert_out_close(out[:, 0], ref)
+
+
+def _assert_within_ulps(got, ref, mant_bits, ulps, what):
+    got, ref = got.double(), ref.double()
+    tol = ref.abs() * (2.0 ** -mant_bits) * ulps + 1e-30
+    bad = (got - ref).abs() > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements beyond {ulps} ulp, worst {(got - ref).abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("dtype,mant,ulps", [(torch.bfloat16, 7, 1), (torch.float16, 10, 1), (torch.float32, 23, 8)])
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("rope", [True, False])
+def test_fused_qk_norm(fd, dtype, mant, ulps, D, rope):
+    """RMS norm of q and k inside the append launch against the float64 oracle: within rounding of the activation
+    dtype (a different summation order cannot be bit-exact), V untouched by the norm, bit-exact."""
+    gen = torch.Generator().manual_seed(D + mant)
+    B, T, Hq, Hkv, P, num_pages = 3, 2, 6, 2, 8, 16
+    lens = [0, 7, 11]
+    q = (torch.randn(B, T, Hq, D, generator=gen) * 3).to(dtype)
+    k = (torch.randn(B, T, Hkv, D, generator=gen) * 0.2).to(dtype)
+    v = torch.randn(B, T, Hkv, D, generator=gen).to(dtype)
+    qw = (1 + 0.3 * torch.randn(D, generator=gen)).to(dtype)
+    kw = (1 + 0.3 * torch.randn(D, generator=gen)).to(dtype)
+    bt = _tables(B, [n + T for n in lens], P, num_pages, gen)
+    kv_lens = torch.tensor(lens, dtype=torch.int32)
+    tab = _cos_sin(D, 64) if rope else None
+    pos = (kv_lens[:, None] + torch.arange(T)).long() if rope else None
+    kc = torch.zeros(num_pages, P, Hkv, D, dtype=dtype)
+    vc = torch.zeros_like(kc)
+
+    q_ref = oracle.ref_rms_norm(q, qw, 1e-6)
+    k_ref = oracle.ref_rms_norm(k, kw, 1e-5)
+    if rope:
+        q_ref, k_ref = oracle.ref_rope(q_ref, tab, pos), oracle.ref_rope(k_ref, tab, pos)
+    ref_k, ref_v = kc.clone(), vc.clone()
+    oracle.ref_kv_append(k_ref, v, ref_k, ref_v, bt, kv_lens)
+
+    g = lambda t: t.to(DEV) if t is not None else None  # noqa: E731
+    kc_g, vc_g = g(kc), g(vc)
+    q_out = fd.rope_kv_append(g(k), g(v), kc_g, vc_g, g(bt), g(kv_lens), cos_sin=g(tab), position_ids=g(pos), q=g(q),
+                              q_norm=(g(qw), 1e-6), k_norm=(g(kw), 1e-5))
+    torch.cuda.synchronize()
+    if rope:
+        # each output mixes two normalised values (each off by up to `ulps`) and is rounded once more: bound the
+        # error by the larger partner of the rotated pair
+        def close(got, ref):
+            got, ref = got.double().reshape(-1, D), ref.double().reshape(-1, D)
+            pair = torch.maximum(ref[:, :D // 2].abs(), ref[:, D // 2:].abs()).repeat(1, 2)
+            return ((got - ref).abs() <= pair * (2.0 ** -mant) * (3 * ulps + 1) + 1e-30).all()
+        assert close(q_out.cpu(), q_ref), "q"
+        assert close(kc_g.cpu(), ref_k), "K cache"
+    else:
+        _assert_within_ulps(q_out.cpu(), q_ref, mant, ulps, "q")
+        _assert_within_ulps(kc_g.cpu(), ref_k, mant, ulps, "K cache")
+    assert torch.equal(vc_g.cpu().view(torch.uint8), ref_v.view(torch.uint8))
+    # q-only call (no append): the same rows
+    q_only = fd.rope_kv_append(None, None, None, None, None, None, cos_sin=g(tab), position_ids=g(pos), q=g(q),
+                               q_norm=(g(qw), 1e-6))
+    torch.cuda.synchronize()
+    assert torch.equal(q_only.cpu().view(torch.uint8), q_out.cpu().view(torch.uint8))

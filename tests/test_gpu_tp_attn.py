@@ -89,10 +89,9 @@ def test_decode_block_steps(fd, cache_kind, qk_norm):
         # oracle from the projected activations (the projections themselves are library GEMMs on both sides)
         qkv = torch.nn.functional.linear(x.to(DEV), attn.wqkv)
         q, k, v = [t.view(B, 1, -1, D) for t in qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)]
-        if qk_norm:
-            q = fd.layers.layer_norm(q.contiguous(), 1e-6, attn.q_norm_w)
-            k = fd.layers.layer_norm(k.contiguous(), 1e-6, attn.k_norm_w)
         q, k, v = q.cpu(), k.cpu(), v.cpu()
+        if qk_norm:
+            q, k = oracle.ref_rms_norm(q, qn, 1e-6), oracle.ref_rms_norm(k, kn, 1e-6)
         q_r, k_r = oracle.ref_rope(q, tab.cpu(), pos), oracle.ref_rope(k, tab.cpu(), pos)
         ref_off = oracle.ref_kv_append(k_r, v, ref_kc, ref_vc, bt_cpu, ref_off, ks_cpu, vs_cpu)
         kf = oracle.dequant_fp8_cache(ref_kc, ks_cpu) if fp8 else ref_kc.float()
@@ -101,7 +100,13 @@ def test_decode_block_steps(fd, cache_kind, qk_norm):
         ref_y = torch.nn.functional.linear(o.view(B, 1, -1), wo.float())
 
         assert torch.equal(cache.get_kv_len().cpu(), ref_off)
-        assert torch.equal(kc.cpu().view(torch.uint8), ref_kc.view(torch.uint8)), f"K cache differs at step {step}"
+        if qk_norm:
+            # the fused norm sums in another order than the float64 oracle: K agrees to rounding, not bit for bit
+            got_k = oracle.dequant_fp8_cache(kc.cpu(), ks_cpu) if fp8 else kc.cpu().float()
+            assert (got_k - kf).abs().max().item() <= (0.13 if fp8 else 0.04), f"K cache differs at step {step}"
+            ref_kc.copy_(kc.cpu())   # continue from the same cache on both sides
+        else:
+            assert torch.equal(kc.cpu().view(torch.uint8), ref_kc.view(torch.uint8)), f"K cache differs at step {step}"
         assert torch.equal(vc.cpu().view(torch.uint8), ref_vc.view(torch.uint8))
         err = (y.float().cpu() - ref_y).abs().max().item()
         assert err <= 3e-2, f"step {step}: max abs err {err}"

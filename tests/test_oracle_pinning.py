@@ -497,3 +497,23 @@ def test_append_capacity_and_fp8():
     # dequantised values are within half an fp8 step (2^-4 relative) of the source
     deq = oracle.dequant_fp8_cache(kc[0:1, 2:3], ks)[0, 0]
     assert ((deq - k[0, 0]).abs() <= 0.0625 * k[0, 0].abs() + 0.01 * 2 ** -9 + 1e-7).all()
+
+
+def test_rms_norm_against_library_and_closed_forms():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 2, 4, 32, generator=g)
+    w = 1 + 0.2 * torch.randn(32, generator=g)
+    got = oracle.ref_rms_norm(x, w, 1e-6)
+    lib = torch.nn.functional.rms_norm(x.view(-1, 32), (32,), weight=w, eps=1e-6).view_as(x)
+    assert (got - lib).abs().max() < 2e-6
+    # eps = 0: invariant under scaling of the row; with w = 1 every output row has RMS 1
+    ones = torch.ones(32)
+    assert torch.allclose(oracle.ref_rms_norm(x * 7.5, ones, 0.0), oracle.ref_rms_norm(x, ones, 0.0), atol=1e-6)
+    assert torch.allclose(oracle.ref_rms_norm(x, ones, 0.0).pow(2).mean(-1), torch.ones(3, 2, 4), atol=1e-5)
+    # constant row c: c / sqrt(c^2 + eps) * w
+    c = torch.full((1, 1, 1, 32), 3.0)
+    assert torch.allclose(oracle.ref_rms_norm(c, w, 1.0), (3.0 / (10.0 ** 0.5)) * w.view(1, 1, 1, 32), atol=1e-6)
+    # rounded once to the activation dtype
+    xb = x.to(torch.bfloat16)
+    assert torch.equal(oracle.ref_rms_norm(xb, w.to(torch.bfloat16), 1e-6),
+                       oracle.ref_rms_norm(xb.double(), w.to(torch.bfloat16).double(), 1e-6).to(torch.bfloat16))

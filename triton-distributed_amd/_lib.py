@@ -53,14 +53,15 @@ class FdParams(Structure):
     ]
 
 
-class FdRope(Structure):
-    """Mirror of ``struct fd_rope``."""
+class FdQkPrep(Structure):
+    """Mirror of ``struct fd_qk_prep``."""
     _fields_ = [
         ("cos_sin", c_void_p), ("stride_cos_sin", c_int64), ("position_ids", c_void_p),
         ("position_dtype", c_int32), ("max_positions", c_int32), ("stride_pos_b", c_int64), ("stride_pos_t", c_int64),
         ("q", c_void_p), ("q_out", c_void_p),
         ("stride_q_b", c_int64), ("stride_q_t", c_int64), ("stride_q_h", c_int64),
         ("stride_qo_b", c_int64), ("stride_qo_t", c_int64), ("stride_qo_h", c_int64),
+        ("q_norm_weight", c_void_p), ("k_norm_weight", c_void_p), ("q_norm_eps", c_float), ("k_norm_eps", c_float),
     ]
 
 
@@ -100,7 +101,7 @@ def load_library(path: str = None) -> ctypes.CDLL:
     lib.fd_kv_append.restype = c_int32
     lib.fd_kv_append.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
-        i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, POINTER(FdRope), POINTER(FdParams)]
+        i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, POINTER(FdQkPrep), POINTER(FdParams)]
     lib.fd_schedule.restype = c_int32
     lib.fd_schedule.argtypes = [c_void_p, c_void_p, c_int32, c_void_p]
     lib.fd_last_error.restype = c_char_p

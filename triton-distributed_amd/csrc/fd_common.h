@@ -93,6 +93,9 @@ struct AppendArgs {
   const void* q;         // nullptr: no query rows
   void* q_out;
   int64_t sq_b, sq_t, sq_h, sqo_b, sqo_t, sqo_h;
+  const void* qn_w;      // nullptr: q is not normalised; else [D] RMS-norm weight in the activation dtype
+  const void* kn_w;
+  float qn_eps, kn_eps;
 };
 
 // ---------------------------------------------------------------- scalar conversions

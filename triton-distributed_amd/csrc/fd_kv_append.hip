@@ -1,5 +1,5 @@
-// Write side of the paged KV cache: rotary embedding of the new tokens' Q and K, and the
-// append of K / V into the page pool (with conversion to the cache's dtype, fp8-e4m3
+// Write side of the paged KV cache: per-head RMS norm and rotary embedding of the new tokens' Q and
+// K, and the append of K / V into the page pool (with conversion to the cache's dtype, fp8-e4m3
 // quantisation included).  One launch covers all of it.
 //
 // A thread owns 8 consecutive elements of the first half of one head row and the matching 8
@@ -91,6 +91,26 @@ __device__ __forceinline__ void rotate8(float* x1, float* x2, const float* cs_ro
   }
 }
 
+// RMS norm of one head row held by `cpr` consecutive lanes (8 + 8 elements each):
+// y = (x * rsqrt(mean(x^2) + eps)) * w in fp32, rounded to the activation dtype.
+template <typename SRC>
+__device__ __forceinline__ void rms_norm_row(float* x1, float* x2, const void* w, float eps, int e0, int half,
+                                             int cpr) {
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss += x1[i] * x1[i] + x2[i] * x2[i];
+  for (int off = 1; off < cpr; off <<= 1) ss += __shfl_xor(ss, off);   // the row's lanes are aligned to cpr
+  const float rstd = 1.0f / sqrtf(ss / (float)(2 * half) + eps);
+  float w1[8], w2[8];
+  load8<SRC>(w, e0, w1);
+  load8<SRC>(w, half + e0, w2);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x1[i] = round_through<SRC>(x1[i] * rstd * w1[i]);
+    x2[i] = round_through<SRC>(x2[i] * rstd * w2[i]);
+  }
+}
+
 template <typename SRC, typename DST>
 __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
   const int cpr = a.D >> 4;                     // threads per head row
@@ -142,6 +162,7 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
     const int64_t src = b * a.sq_b + t * a.sq_t + h * a.sq_h;
     load8<SRC>(a.q, src + e0, x1);
     load8<SRC>(a.q, src + half + e0, x2);
+    if (a.qn_w) rms_norm_row<SRC>(x1, x2, a.qn_w, a.qn_eps, e0, half, cpr);
     if (cs_row) rotate8<SRC>(x1, x2, cs_row, e0, half);
     const int64_t dst = b * a.sqo_b + t * a.sqo_t + h * a.sqo_h;
     store8<SRC>(a.q_out, dst + e0, x1, 1.f);
@@ -177,6 +198,7 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
     const int64_t src = b * a.skn_b + t * a.skn_t + h * a.skn_h;
     load8<SRC>(a.k_new, src + e0, x1);
     load8<SRC>(a.k_new, src + half + e0, x2);
+    if (a.kn_w) rms_norm_row<SRC>(x1, x2, a.kn_w, a.kn_eps, e0, half, cpr);
     if (cs_row) rotate8<SRC>(x1, x2, cs_row, e0, half);
     const float scale = ElemBytes<DST>::v == 1 ? a.k_scale[h] : 1.f;
     const int64_t dst = trow * a.sk_t + h * a.sk_h;

@@ -19,16 +19,18 @@ from typing import Optional, Tuple, Union
 
 import torch
 
-from .._lib import FdParams, FdRope, check, fd_dtype_of, load_library, stream_handle
+from .._lib import FdParams, FdQkPrep, check, fd_dtype_of, load_library, stream_handle
 from .flash_decode import _decode, _require_cuda
 
 
-def _rope_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdRope:
+def _prep_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdQkPrep:
+    r = FdQkPrep()
+    if cos_sin is None:
+        return r
     assert cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.stride(1) == 1
     assert cos_sin.shape[1] == head_dim, "cos_sin rows hold head_dim/2 cosines then head_dim/2 sines"
     assert position_ids.dim() == 2 and tuple(position_ids.shape) == (bsz, seq)
     assert position_ids.dtype in (torch.int32, torch.int64)
-    r = FdRope()
     r.cos_sin = cos_sin.data_ptr()
     r.stride_cos_sin = cos_sin.stride(0)
     r.position_ids = position_ids.data_ptr()
@@ -44,12 +46,15 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
                    seq_order_out: Optional[torch.Tensor] = None,
                    k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
                    cos_sin: Optional[torch.Tensor] = None, position_ids: Optional[torch.Tensor] = None,
-                   q: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None, stream=None):
+                   q: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None,
+                   q_norm: Optional[Tuple[torch.Tensor, float]] = None,
+                   k_norm: Optional[Tuple[torch.Tensor, float]] = None, stream=None):
     """Appends ``k_new`` / ``v_new`` ``[B, T, Hkv, D]`` at positions ``kv_lens[b] .. +T-1`` of the paged pool.
 
     With ``cos_sin`` (fp32 ``[max_pos, D]``) and ``position_ids`` (``[B, T]`` int32/int64) K is rotated before it
     is stored and ``q`` ``[B, T, Hq, D]`` (if given) is rotated into ``q_out`` (default: a new tensor; may be
-    ``q``) in the same launch.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
+    ``q``) in the same launch.  ``q_norm`` / ``k_norm`` = ``(weight [D], eps)`` apply the per-head RMS norm of the
+    reference's block (tp_attn.py:252-258) to q / k before the rotation.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
     ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out`` (int32 ``[B]``, not ``kv_lens``) receives
     the grown lengths; ``seq_order_out`` (int32 ``[B]``, ``B <= 4096``) the longest-first issue order for the
     decode that follows (what ``schedule_sequences`` would compute, without a launch of its own).  Returns
@@ -95,8 +100,15 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
         sk, sv = (k_cache.stride(1), k_cache.stride(2)), (v_cache.stride(1), v_cache.stride(2))
         sbt = block_table.stride(0)
     rope = None
-    if cos_sin is not None:
-        rope = _rope_struct(cos_sin, position_ids, head_dim, bsz, seq)
+    if cos_sin is not None or q_norm is not None or k_norm is not None:
+        rope = _prep_struct(cos_sin, position_ids, head_dim, bsz, seq)
+        for name, norm in (("q", q_norm), ("k", k_norm)):
+            if norm is not None:
+                w, eps = norm
+                _require_cuda(w)
+                assert w.dtype == src.dtype and w.is_contiguous() and w.numel() == head_dim
+                setattr(rope, name + "_norm_weight", w.data_ptr())
+                setattr(rope, name + "_norm_eps", float(eps))
         if q is not None:
             assert q.dim() == 4 and q.shape[0] == bsz and q.shape[1] == seq and q.shape[3] == head_dim
             assert q.dtype == src.dtype and q.stride(-1) == 1
@@ -107,7 +119,7 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
             rope.stride_q_b, rope.stride_q_t, rope.stride_q_h = q.stride()[:3]
             rope.stride_qo_b, rope.stride_qo_t, rope.stride_qo_h = q_out.stride()[:3]
     elif q is not None:
-        raise RuntimeError("rope_kv_append: q is only processed together with cos_sin / position_ids")
+        raise RuntimeError("rope_kv_append: q is only processed together with cos_sin / position_ids or a norm")
     check(lib.fd_kv_append(
         stream_handle(stream, src.device.index), ptr(k_new), ptr(v_new), ptr(k_cache), ptr(v_cache), ptr(block_table),
         ptr(kv_lens), ptr(kv_lens_out), ptr(seq_order_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
@@ -151,7 +163,8 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
                             cache_leftpad=None, block_table=None, softmax_scale=None, causal=False,
                             window_size=(-1, -1), softcap=0.0, rotary_interleaved=True, alibi_slopes=None,
                             num_splits=0, return_softmax_lse=False, *, cos_sin_cache=None, position_ids=None,
-                            k_scale=None, v_scale=None, kv_lens_out=None, stream=None, **decode_kw):
+                            k_scale=None, v_scale=None, kv_lens_out=None, q_norm=None, k_norm=None, stream=None,
+                            **decode_kw):
     """Decode-step drop-in for the flash-attn call of the reference's attention block (tp_attn.py:268-269).
 
     ``q [B, 1, Hq, D]``; ``k_cache`` / ``v_cache`` either dense ``[B_cache, L, Hkv, D]`` (the reference's
@@ -162,7 +175,8 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
     ``[B, Hq, 1]`` fp32 with ``return_softmax_lse``).
 
     Beyond flash-attn: ``cos_sin_cache`` + ``position_ids`` (the reference's rotary format) rotate q and k
-    on the way in, in the append launch; ``k_scale`` / ``v_scale`` select an fp8-e4m3 cache;
+    on the way in, in the append launch, after the per-head RMS norms ``q_norm`` / ``k_norm`` =
+    ``(weight, eps)``; ``k_scale`` / ``v_scale`` select an fp8-e4m3 cache;
     ``kv_lens_out`` receives ``cache_seqlens + T``.  ``num_splits`` 0 lets the library choose.
     Not covered, and refused: more than one query token, flash-attn's own rotary arguments, left padding,
     sliding windows and ALiBi.
@@ -199,15 +213,17 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
         if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw:
             # the append launch also ranks the sequences (longest first) for the decode's issue order
             decode_kw["seq_order"] = torch.empty_like(cache_seqlens)
+        prep_q = cos_sin_cache is not None or q_norm is not None
         q_rot = rope_kv_append(k, v, k_cache, v_cache, block_table, cache_seqlens, kv_lens_out=kv_lens_out,
-                               seq_order_out=decode_kw.get("seq_order"), k_scale=k_scale, v_scale=v_scale, cos_sin=cos_sin_cache, position_ids=position_ids,
-                               q=q if cos_sin_cache is not None else None, stream=stream)
+                               seq_order_out=decode_kw.get("seq_order"), k_scale=k_scale, v_scale=v_scale,
+                               cos_sin=cos_sin_cache, position_ids=position_ids, q=q if prep_q else None,
+                               q_norm=q_norm, k_norm=k_norm, stream=stream)
         if q_rot is None:
             q_rot = q
         kv_lens = kv_lens_out
-    elif cos_sin_cache is not None:
+    elif cos_sin_cache is not None or q_norm is not None:
         q_rot = rope_kv_append(None, None, None, None, None, None, cos_sin=cos_sin_cache, position_ids=position_ids,
-                               q=q, stream=stream)
+                               q=q, q_norm=q_norm, stream=stream)
 
     out = torch.empty_like(q)
     lse = torch.empty((bsz, q_heads), dtype=torch.float32, device=dev) if return_softmax_lse else None

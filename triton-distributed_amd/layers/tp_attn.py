@@ -3,7 +3,7 @@
 ``TP_Attn`` keeps the reference's constructor, parameter layout and forward signature
 (``python/triton_dist/layers/amd/tp_attn.py:171-308``): fused QKV projection, optional per-head RMS norm of
 q and k, rotary embedding, cache update, attention, output projection.  What changes is the middle: the
-rotary embedding of q and k and the cache update are ONE launch of the append kernel, and the attention is
+q/k norms, the rotary embedding of q and k and the cache update are ONE launch of the append kernel, and the attention is
 the split-KV decode of this package instead of the flash-attn package (tp_attn.py:262-269).  The two
 projections stay plain ``torch.nn.functional.linear`` calls (hipBLASLt), as in the reference's
 ``torch_fwd``.
@@ -88,15 +88,14 @@ class TP_Attn:
         q = q.view(bsz, q_len, -1, self.head_dim)
         k = k.view(bsz, q_len, -1, self.head_dim)
         v = v.view(bsz, q_len, -1, self.head_dim)
-        if hasattr(self, "q_norm_eps"):
-            q = layer_norm(q.contiguous(), self.q_norm_eps, self.q_norm_w)
-        if hasattr(self, "k_norm_eps"):
-            k = layer_norm(k.contiguous(), self.k_norm_eps, self.k_norm_w)
+        # the per-head RMS norms of q and k (tp_attn.py:252-258) run inside the append launch
+        q_norm = (self.q_norm_w, self.q_norm_eps) if hasattr(self, "q_norm_eps") else None
+        k_norm = (self.k_norm_w, self.k_norm_eps) if hasattr(self, "k_norm_eps") else None
         k_cache, v_cache, kv_offset = kv_cache.update_kv_cache(k, v, layer_idx)
         out = flash_attn_with_kvcache(q, k_cache, v_cache, k=k, v=v, cache_seqlens=kv_offset,
                                       block_table=kv_cache.block_table, causal=True, cos_sin_cache=cos_sin_cache,
                                       position_ids=position_ids, k_scale=kv_cache.k_scale, v_scale=kv_cache.v_scale,
-                                      **decode_kw)
+                                      q_norm=q_norm, k_norm=k_norm, **decode_kw)
         return nn.functional.linear(out.view(bsz, q_len, -1), self.wo)
 
     torch_fwd = fwd
