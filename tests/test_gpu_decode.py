@@ -51,6 +51,24 @@ def test_reference_grid_fp16(fd, kv_lens, num_heads, head_size, block_size, soft
     assert_lse_close(lse, ref_lse)
 
 
+# ---- head_dim 64 (its own MFMA kernel for groups >= 4; VALU otherwise)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("num_heads", [(32, 8), (64, 8), (6, 1), (16, 16), (28, 4), (32, 1)])
+@pytest.mark.parametrize("block_size,soft_cap", [(1, 0), (16, 0), (16, 30), (7, 50)])
+def test_head_dim_64(fd, dtype, num_heads, block_size, soft_cap):
+    wl = _grid_workload(fd, [1320, 18, 463, 1, 0, 64, 65, 2500], num_heads, 64, block_size, dtype, soft_cap, seed=11)
+    out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+    if num_heads[0] // num_heads[1] >= 4:      # both kernels exist for this shape: they agree with each other too
+        out_v, lse_v = run_decode(fd, wl, path="valu")
+        assert_out_close(out_v, ref)
+        out_m, lse_m = run_decode(fd, wl, path="mfma", waves_per_block=2, plan_splits=False)
+        assert_out_close(out_m, ref)
+        assert_lse_close(lse_m, ref_lse)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("num_heads", [(16, 16), (8, 4), (32, 8), (64, 8), (6, 1), (32, 2), (3, 1)])
 @pytest.mark.parametrize("block_size", [1, 16, 7])
