@@ -301,7 +301,7 @@ def main():
     # per 32 tokens of one (sequence, KV head, block of <=16 query heads) 16 MFMAs of 16x16x32 (16 384 flop each);
     # the committed counter run (profiles/*mfma_utilisation.md) reads exactly this number.
     G = Hq // wl.k_cache.shape[2]
-    if D == 128 and G >= 4 and args.path != "valu" and wl.q.dtype != torch.float32:
+    if D == 128 and args.path != "valu" and wl.q.dtype != torch.float32:
         tokens = int(wl_cpu.kv_lens.sum())
         nhb = -(-G // 16)
         issued = tokens * wl.k_cache.shape[2] * nhb * 16 * 16384 / 32

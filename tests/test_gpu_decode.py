@@ -51,7 +51,7 @@ def test_reference_grid_fp16(fd, kv_lens, num_heads, head_size, block_size, soft
     assert_lse_close(lse, ref_lse)
 
 
-# ---- head_dim 64 (its own MFMA kernel for groups >= 4; VALU otherwise)
+# ---- head_dim 64 (its own MFMA kernel)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("num_heads", [(32, 8), (64, 8), (6, 1), (16, 16), (28, 4), (32, 1)])
 @pytest.mark.parametrize("block_size,soft_cap", [(1, 0), (16, 0), (16, 30), (7, 50)])
@@ -61,7 +61,7 @@ def test_head_dim_64(fd, dtype, num_heads, block_size, soft_cap):
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
-    if num_heads[0] // num_heads[1] >= 4:      # both kernels exist for this shape: they agree with each other too
+    if num_heads[0] // num_heads[1] <= 16:     # both kernels exist for this shape: they agree with each other too
         out_v, lse_v = run_decode(fd, wl, path="valu")
         assert_out_close(out_v, ref)
         out_m, lse_m = run_decode(fd, wl, path="mfma", waves_per_block=2, plan_splits=False)
@@ -410,8 +410,8 @@ def test_errors_are_reported_not_fatal(fd):
     with pytest.raises(AssertionError):   # head-dim mismatch: the reference asserts too (flash_decode.py:767)
         fd.gqa_fwd_batch_decode(wl.q[:, :, :64], wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0)
     with pytest.raises(RuntimeError, match="MFMA path"):
-        fd.gqa_fwd_batch_decode(wl.q[:, :8], wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0,
-                                path="mfma")   # group 1 cannot take the MFMA path
+        fd.gqa_fwd_batch_decode(wl.q.float(), wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0,
+                                path="mfma")   # an fp32 query cannot take the MFMA path
     with pytest.raises(RuntimeError, match="Unsupported data type"):
         fd.gqa_fwd_batch_decode(wl.q.double(), wl.k_cache, wl.v_cache, None, [1], wl.kv_lens, wl.block_table, 1.0)
     # and the library still works afterwards

@@ -182,7 +182,8 @@ def test_split_plan_policy(fd):
     assert plan(64, 32, 8, 32, 2048) == 8          # config 4: <= 4096 tokens per split of a full-length sequence
     assert plan(32, 64, 8, 64, 1024, kv=L.FD_FP8_E4M3) == 4
     assert plan(8, 32, 8, 32, 512, D=256) == 8     # head_dim 256 has an MFMA kernel too
-    assert plan(8, 8, 8, 32, 512) == 8             # VALU path (MHA): 2048 waves with 4 waves per (head, split)
+    assert plan(8, 8, 8, 32, 512) == 8             # MHA runs on the MFMA kernels too
+    assert plan(8, 8, 8, 32, 512, kv=L.FD_F32) == 8  # VALU path (fp32 cache): 2048 waves with 4 waves per (head, split)
     assert plan(2, 8, 8, 32, 512) == 32
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1

@@ -1,8 +1,8 @@
 // Split-KV GQA paged decode on MFMA (gfx950), head_dim 128, 16-bit KV cache.
 //
 // Replaces kernel_gqa_fwd_batch_decode_split_kv
-// (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) for GQA groups
-// of at least 4 query heads per KV head.
+// (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) for every GQA group
+// (the query heads of a KV head are padded to blocks of 16, the MFMA N).
 //
 // Decomposition: one workgroup per (sequence, split, KV head, block of <=16
 // query heads); its W waves take contiguous runs of 32-token tiles of the split

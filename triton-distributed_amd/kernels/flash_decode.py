@@ -49,7 +49,7 @@ def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size,
     """Meta-parameters of the split kernel, the counterpart of ``get_triton_split_kv_algo_info``
     (flash_decode.py:103-109): what the gfx950 kernels use instead of BLOCK_N/BLOCK_H/num_warps."""
     group = q_heads // kv_heads
-    mfma = q_head_dim in (64, 128, 256) and group >= 4
+    mfma = q_head_dim in (64, 128, 256)   # 16-bit / fp8 caches; fp32 caches run on the VALU kernel
     return {
         "kv_group_num": group, "q_head_num": q_heads, "NUM_KV_SPLITS": split_kv, "PAGE_SIZE": page_size,
         "soft_cap": soft_cap, "K_DIM": q_head_dim, "V_DIM": v_head_dim,
