@@ -61,16 +61,17 @@ def test_head_dim_64(fd, dtype, num_heads, block_size, soft_cap):
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
-    if num_heads[0] // num_heads[1] <= 16:     # both kernels exist for this shape: they agree with each other too
-        out_v, lse_v = run_decode(fd, wl, path="valu")
-        assert_out_close(out_v, ref)
-        out_m, lse_m = run_decode(fd, wl, path="mfma", waves_per_block=2, plan_splits=False)
-        assert_out_close(out_m, ref)
-        assert_lse_close(lse_m, ref_lse)
+    # both kernels exist for every shape here: each agrees with the oracle when forced
+    out_v, lse_v = run_decode(fd, wl, path="valu")
+    assert_out_close(out_v, ref)
+    out_m, lse_m = run_decode(fd, wl, path="mfma", waves_per_block=2, plan_splits=False)
+    assert_out_close(out_m, ref)
+    assert_lse_close(lse_m, ref_lse)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("num_heads", [(16, 16), (8, 4), (32, 8), (64, 8), (6, 1), (32, 2), (3, 1)])
+@pytest.mark.parametrize("num_heads", [(16, 16), (8, 4), (32, 8), (64, 8), (6, 1), (32, 2), (3, 1), (20, 1), (48, 2),
+                                       (33, 1)])
 @pytest.mark.parametrize("block_size", [1, 16, 7])
 def test_other_dtypes_and_groups(fd, dtype, num_heads, block_size):
     wl = _grid_workload(fd, [1320, 18, 463, 1, 70], num_heads, 128, block_size, dtype, 0, seed=3)

@@ -43,13 +43,14 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
 }
 
 // Shapes the MFMA split kernels are built for: head_dim 128 with a 16-bit or fp8-e4m3 cache, head_dim 64 or 256 with
-// a 16-bit cache; any GQA group that is <= 16 or a multiple of 16 (blocks of 16 query heads, padded: even with one
+// a 16-bit cache; any GQA group (blocks of 16 query heads, the last one padded: even with one
 // query head per KV head the MFMA kernels stream faster than the VALU kernel, 46.1 vs 50.2 us on config 2's shape as MHA,
 // 46.1 vs 78.9 us with 3 query heads per KV head).
 bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
   const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
   const bool dim_ok = (head_dim == 128 && (kv16 || kv_dtype == FD_FP8_E4M3)) || ((head_dim == 64 || head_dim == 256) && kv16);
-  return dim_ok && (group <= 16 || group % 16 == 0);
+  (void)group;
+  return dim_ok;
 }
 
 // Launch-shape policy, from sweeps on one MI355X (256 CUs): the MFMA kernels stream best with about
@@ -175,8 +176,8 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs head_dim 128 (or 64 / 256 with a 16-bit cache), a group <= 16 or a multiple of "
-                "16, a 16-bit query with a KV cache of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
+                "%s: MFMA path needs head_dim 128 (or 64 / 256 with a 16-bit cache), a 16-bit query with a KV cache "
+                "of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
