@@ -45,6 +45,9 @@ def parse_args():
                     help="skip the timing of the step before the decode (rotary + KV append)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
+    ap.add_argument("--shape", default=None,
+                    help="B,kv_len,Hq,Hkv,D,P[,bf16|fp16|fp8]: a uniform batch of another shape instead of a BASELINE "
+                         "config (secondary measurements: other head dims, groups, batch sizes)")
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: a kernel of known traffic against which "
                          "a counter run (FETCH_SIZE / WRITE_SIZE) of this same command is scaled")
@@ -154,7 +157,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    wl_cpu = fd.utils.make_config5_bf16_twin() if args.bf16_twin else fd.utils.make_config(args.config)
+    if args.shape:
+        f = args.shape.split(",")
+        B_, n_, hq_, hkv_, d_, p_ = (int(x) for x in f[:6])
+        kind = f[6] if len(f) > 6 else "bf16"
+        wl_cpu = fd.utils.make_paged_workload(
+            f"shape_b{B_}_kv{n_}_hq{hq_}_hkv{hkv_}_d{d_}_p{p_}_{kind}", [n_] * B_, hq_, hkv_, d_, p_,
+            torch.float16 if kind == "fp16" else torch.bfloat16, 32, 2000, fp8_kv=kind == "fp8")
+    elif args.bf16_twin:
+        wl_cpu = fd.utils.make_config5_bf16_twin()
+    else:
+        wl_cpu = fd.utils.make_config(args.config)
     wl = wl_cpu.to(dev)
     B, Hq, D = wl.q.shape
     S = args.kv_split or wl.kv_split
