@@ -17,6 +17,7 @@ namespace {
 
 constexpr int kCombineThreads = 256;
 constexpr int kMaxPartials = 1024;  // LSEs staged in LDS per pass
+constexpr int kPrefetch = 8;        // partial rows a thread requests before the weights are known
 
 template <int D>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const CombineArgs a) {
@@ -33,8 +34,12 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   const int NP = S + a.num_extra;
   const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
 
+  // Partials written by this library's split kernel in the same call: every slot holds defined values (an
+  // empty split is out = 0, lse = -inf), so validity needs no kv_lens and rows may be read before their weights
+  // are known.
+  const bool own = a.all_slots_written && a.mode != FD_COMBINE_RANK;
   int kv_len = 0, per = 0;
-  if (a.mode != FD_COMBINE_RANK) {
+  if (a.mode != FD_COMBINE_RANK && !own) {
     kv_len = max(a.seqlens[b], 0);
     per = (kv_len + S - 1) / S;
   }
@@ -43,7 +48,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
     if (s >= S) return a.extra_lse[((int64_t)(s - S) * a.batch + b) * a.Hq + h];  // extras: always valid
     if (a.mode == FD_COMBINE_RANK) {
       if (a.seqlens[(int64_t)s * a.batch + b] <= 0) return -INFINITY;
-    } else if ((int64_t)per * s >= kv_len) {  // empty split range
+    } else if (!own && (int64_t)per * s >= kv_len) {  // empty split range
       return -INFINITY;
     }
     if (a.mid_lse) return a.mid_lse[((int64_t)b * a.Hq + h) * S + s];
@@ -53,43 +58,67 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   const int r = tid / CG;
   const int c = tid - r * CG;
   const bool vec_mid = a.mid_dtype == FD_F32 && a.vec_mid;
+  auto load_row = [&](int s) -> f32x4 {   // this thread's 4 columns of partial s
+    f32x4 o;
+    if (s < S) {
+      const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
+      if (vec_mid) {
+        o = *(const f32x4*)((const float*)a.mid_o + off);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.mid_o, off + k, a.mid_dtype);
+      }
+    } else {
+      const int64_t off = (((int64_t)(s - S) * a.batch + b) * a.Hq + h) * D + 4 * c;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.extra_out, off + k, a.out_dtype);
+    }
+    return o;
+  };
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float M = -INFINITY;  // running max over the passes (one pass unless NP > kMaxPartials)
   float L = 0.f;        // sum of the weights of this thread's rows
 
-  for (int p0 = 0; p0 < NP; p0 += kMaxPartials) {
-    const int cnt = min(kMaxPartials, NP - p0);
-    __syncthreads();
-    for (int i = tid; i < cnt; i += kCombineThreads) s_lse[i] = partial_lse(p0 + i);
-    __syncthreads();
-    float m_pass = -INFINITY;
-    for (int i = 0; i < cnt; ++i) m_pass = fmaxf(m_pass, s_lse[i]);
-    const float m_new = fmaxf(M, m_pass);
-    if (m_new == -INFINITY) continue;  // nothing valid so far (uniform)
-    const float resc = __expf(M - m_new);  // 0 on the first valid pass
-    acc *= resc;
-    L *= resc;
-    M = m_new;
-    for (int i = r; i < cnt; i += ROWS) {
-      const float wgt = __expf(s_lse[i] - M);
-      if (wgt == 0.f) continue;
-      const int s = p0 + i;
-      f32x4 o;
-      if (s < S) {
-        const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
-        if (vec_mid) {
-          o = *(const f32x4*)((const float*)a.mid_o + off);
-        } else {
+  if (own && NP <= ROWS * kPrefetch) {
+    // one dependent round trip: the rows are requested together with the LSEs
+    f32x4 pre[kPrefetch];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.mid_o, off + k, a.mid_dtype);
-        }
-      } else {
-        const int64_t off = (((int64_t)(s - S) * a.batch + b) * a.Hq + h) * D + 4 * c;
+    for (int p = 0; p < kPrefetch; ++p) {
+      const int s = r + p * ROWS;
+      pre[p] = s < NP ? load_row(s) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int i = tid; i < NP; i += kCombineThreads) s_lse[i] = partial_lse(i);
+    __syncthreads();
+    for (int i = 0; i < NP; ++i) M = fmaxf(M, s_lse[i]);
+    if (M > -INFINITY) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.extra_out, off + k, a.out_dtype);
+      for (int p = 0; p < kPrefetch; ++p) {
+        const int s = r + p * ROWS;
+        const float wgt = s < NP ? __expf(s_lse[s] - M) : 0.f;
+        acc += pre[p] * wgt;
+        L += wgt;
       }
-      acc += o * wgt;
-      L += wgt;
+    }
+  } else {
+    for (int p0 = 0; p0 < NP; p0 += kMaxPartials) {
+      const int cnt = min(kMaxPartials, NP - p0);
+      __syncthreads();
+      for (int i = tid; i < cnt; i += kCombineThreads) s_lse[i] = partial_lse(p0 + i);
+      __syncthreads();
+      float m_pass = -INFINITY;
+      for (int i = 0; i < cnt; ++i) m_pass = fmaxf(m_pass, s_lse[i]);
+      const float m_new = fmaxf(M, m_pass);
+      if (m_new == -INFINITY) continue;  // nothing valid so far (uniform)
+      const float resc = __expf(M - m_new);  // 0 on the first valid pass
+      acc *= resc;
+      L *= resc;
+      M = m_new;
+      for (int i = r; i < cnt; i += ROWS) {
+        const float wgt = __expf(s_lse[i] - M);
+        if (wgt == 0.f) continue;
+        acc += load_row(p0 + i) * wgt;
+        L += wgt;
+      }
     }
   }
   *(f32x4*)&s_acc[r][4 * c] = acc;
