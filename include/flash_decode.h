@@ -93,6 +93,9 @@ typedef struct fd_params {
   const float* v_scale;     /* [Hkv]                                               */
   int32_t path;             /* fd_path                                             */
   int32_t waves_per_block;  /* 0 = choose; else 1, 2, 4 or 8 wave64 per workgroup  */
+  const int32_t* seq_order_lens; /* NULL, or [batch] with seq_order: kv_lens[seq_order[r]]
+                               at index r (fd_kv_append writes it), so that a workgroup
+                               fetches its sequence and its length in one round trip */
 } fd_params;
 
 /*
@@ -261,9 +264,11 @@ typedef struct fd_qk_prep {
  *                contiguous, 16-byte aligned rows.  Both NULL: only prep->q is processed.
  *  kv_lens       [batch] tokens already in the cache (not modified)
  *  kv_lens_out   NULL, or [batch] (not kv_lens itself): min(kv_lens[b] + new_tokens, capacity)
- *  seq_order_out NULL, or [batch] int32 (batch <= 4096): what fd_schedule would return for
- *                kv_lens_out -- the issue order for the decode that follows, computed by a few
- *                trailing workgroups of this launch instead of a launch of its own
+ *  seq_order_out NULL, or [2 * batch] int32 (batch <= 4096): entries [0, batch) are what
+ *                fd_schedule would return for kv_lens_out -- the issue order for the decode that
+ *                follows, computed by a few trailing workgroups of this launch instead of a
+ *                launch of its own -- and entries [batch, 2 * batch) are kv_lens_out in that
+ *                order (params->seq_order_lens of the decode)
  *  A token whose position is at or beyond max_pages_per_seq * page_size is not written.
  */
 FD_API int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cache, void* v_cache,

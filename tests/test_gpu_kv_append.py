@@ -288,14 +288,15 @@ def test_append_also_ranks_sequences(fd):
     kc = torch.zeros(B * 3, P, Hkv, D, dtype=torch.bfloat16, device=DEV)
     vc = torch.zeros_like(kc)
     grown = torch.empty(B, dtype=torch.int32, device=DEV)
-    order = torch.full((B,), -1, dtype=torch.int32, device=DEV)
+    order = torch.full((2, B), -1, dtype=torch.int32, device=DEV)
     fd.paged_kv_append(k, k, kc, vc, bt, lens.to(DEV), kv_lens_out=grown, seq_order_out=order)
     want = fd.schedule_sequences(grown)
     torch.cuda.synchronize()
     assert torch.equal(grown.cpu(), (lens + 2).clamp(max=48))
-    assert torch.equal(order.cpu(), want.cpu())
+    assert torch.equal(order[0].cpu(), want.cpu())
     ref = sorted(range(B), key=lambda i: (-int(grown[i]), i))
-    assert order.cpu().tolist() == ref
+    assert order[0].cpu().tolist() == ref
+    assert torch.equal(order[1].cpu(), grown.cpu()[order[0].cpu().long()])      # the lengths in issue order
 
     # the decode-step call: ragged batch of 24 sequences, oracle on the CPU
     B = 24
@@ -314,7 +315,7 @@ def test_append_also_ranks_sequences(fd):
     real = fd.kernels.kv_append._decode
 
     def spy(*a, **kw):
-        seen["order"] = kw.get("seq_order")
+        seen["order"], seen["lens"] = kw.get("seq_order"), kw.get("seq_order_lens")
         return real(*a, **kw)
     fd.kernels.kv_append._decode = spy
     try:
@@ -325,6 +326,7 @@ def test_append_also_ranks_sequences(fd):
     torch.cuda.synchronize()
     assert seen["order"] is not None
     assert seen["order"].cpu().tolist() == sorted(range(B), key=lambda i: (-int(new_lens[i]), i))
+    assert seen["lens"].cpu().tolist() == sorted(new_lens.tolist(), reverse=True)
     assert_out_close(out[:, 0], ref)
 
 

@@ -154,7 +154,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   SplitArgs a;
   memset(&a, 0, sizeof(a));
   a.q = q; a.k = k_cache; a.v = v_cache; a.out = out_split; a.lse = lse_split;
-  a.bt = block_table; a.kv_lens = kv_lens; a.order = seq_order;
+  a.bt = block_table; a.kv_lens = kv_lens; a.order = seq_order; a.order_lens = seq_order ? p->seq_order_lens : nullptr;
   a.k_scale = p->k_scale; a.v_scale = p->v_scale;
   a.sq_b = stride_q_bs; a.sq_h = stride_q_h; a.sk_t = stride_k_tok; a.sk_h = stride_k_h;
   a.sv_t = stride_v_tok; a.sv_h = stride_v_h; a.so_b = stride_o_bs; a.so_h = stride_o_h; a.so_s = stride_o_split;

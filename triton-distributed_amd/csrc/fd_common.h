@@ -32,6 +32,7 @@ struct SplitArgs {
   const int32_t* bt;
   const int32_t* kv_lens;
   const int32_t* order;  // nullptr: identity
+  const int32_t* order_lens;  // nullptr, or kv_lens[order[r]] at index r
   const float* k_scale;
   const float* v_scale;
   int64_t sq_b, sq_h, sk_t, sk_h, sv_t, sv_h, so_b, so_h, so_s, sbt;
@@ -197,7 +198,7 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   int b = a.order ? a.order[r] : r;
   w.b = min(max(b, 0), a.batch - 1);
   int64_t cap = (int64_t)a.max_pages * a.P;
-  int64_t len = a.kv_lens[w.b];
+  int64_t len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
   // per = ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)

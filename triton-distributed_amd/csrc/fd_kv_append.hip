@@ -136,6 +136,7 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
       rank += (other > mine) || (other == mine && j < i);
     }
     a.seq_order[rank] = i;
+    a.seq_order[a.batch + rank] = (int32_t)mine;   // the lengths in issue order, for the decode's prologue
     return;
   }
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;

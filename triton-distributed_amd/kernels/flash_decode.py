@@ -16,6 +16,8 @@ Keyword-only additions that the reference does not have (all default off):
                   the combine, standing in for what other sequence-parallel ranks
                   would contribute
   seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences
+  seq_order_lens  int32 [B], with ``seq_order``: ``kv_lens[seq_order]`` (``rope_kv_append`` writes both), which
+                  saves a workgroup one dependent load before it can start
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
   plan_splits     True (default): when ``output_split`` is not supplied, ``kv_split`` is an upper bound
                   and the library uses ``fd_plan_splits`` splits (same result, fewer workgroup prologues
@@ -88,7 +90,7 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 
 
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
-                 waves_per_block) -> FdParams:
+                 waves_per_block, seq_order_lens=None) -> FdParams:
     p = FdParams()
     p.q_heads = q.shape[1]
     p.kv_heads = k_cache.shape[2]
@@ -106,12 +108,13 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
     p.v_scale = v_scale.data_ptr() if v_scale is not None else None
     p.path = _PATHS[path]
     p.waves_per_block = waves_per_block
+    p.seq_order_lens = seq_order_lens.data_ptr() if seq_order_lens is not None else None
     return p
 
 
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
-            stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True):
+            seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -175,8 +178,11 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     else:
         assert output_combine.shape[-1] >= out_cols and output_combine.stride(-1) == 1
 
+    if seq_order_lens is not None:
+        assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
+        assert seq_order_lens.numel() == batch
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
-                     v_scale, path, waves_per_block)
+                     v_scale, path, waves_per_block, seq_order_lens)
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:

@@ -56,8 +56,9 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
     ``q``) in the same launch.  ``q_norm`` / ``k_norm`` = ``(weight [D], eps)`` apply the per-head RMS norm of the
     reference's block (tp_attn.py:252-258) to q / k before the rotation.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
     ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out`` (int32 ``[B]``, not ``kv_lens``) receives
-    the grown lengths; ``seq_order_out`` (int32 ``[B]``, ``B <= 4096``) the longest-first issue order for the
-    decode that follows (what ``schedule_sequences`` would compute, without a launch of its own).  Returns
+    the grown lengths; ``seq_order_out`` (int32 ``[2, B]``, ``B <= 4096``) the longest-first issue order for the
+    decode that follows (row 0: what ``schedule_sequences`` would compute, without a launch of its own) and the
+    grown lengths in that order (row 1: the decode's ``seq_order_lens``).  Returns
     ``q_out`` (or ``None`` without ``q``).
     """
     lib = load_library()
@@ -90,7 +91,8 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
         if kv_lens_out is not None:
             assert kv_lens_out.dtype == torch.int32 and kv_lens_out.is_contiguous() and kv_lens_out.numel() == bsz
         if seq_order_out is not None:
-            assert seq_order_out.dtype == torch.int32 and seq_order_out.is_contiguous() and seq_order_out.numel() == bsz
+            assert seq_order_out.dtype == torch.int32 and seq_order_out.is_contiguous()
+            assert seq_order_out.numel() == 2 * bsz
         p.page_size = page_size
         p.num_pages = k_cache.shape[0]
         p.max_pages_per_seq = block_table.shape[1]
@@ -210,12 +212,14 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
         assert v is not None
         if kv_lens_out is None:
             kv_lens_out = torch.empty_like(cache_seqlens)
+        order = None
         if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw:
             # the append launch also ranks the sequences (longest first) for the decode's issue order
-            decode_kw["seq_order"] = torch.empty_like(cache_seqlens)
+            order = torch.empty((2, bsz), dtype=torch.int32, device=dev)
+            decode_kw["seq_order"], decode_kw["seq_order_lens"] = order[0], order[1]
         prep_q = cos_sin_cache is not None or q_norm is not None
         q_rot = rope_kv_append(k, v, k_cache, v_cache, block_table, cache_seqlens, kv_lens_out=kv_lens_out,
-                               seq_order_out=decode_kw.get("seq_order"), k_scale=k_scale, v_scale=v_scale,
+                               seq_order_out=order, k_scale=k_scale, v_scale=v_scale,
                                cos_sin=cos_sin_cache, position_ids=position_ids, q=q if prep_q else None,
                                q_norm=q_norm, k_norm=k_norm, stream=stream)
         if q_rot is None:
