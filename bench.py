@@ -31,7 +31,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE.json configs, 1-based (2 = Llama-3-8B shape)")
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (2 = Llama-3-8B shape, the one the metric is quoted on)")
     ap.add_argument("--pools", type=int, default=4, help="independent KV pools the steps rotate over")
     ap.add_argument("--variant", default="plain", choices=["plain", "persistent"])
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
     ap.add_argument("--bf16-twin", action="store_true", help="config 5's shape with a bf16 cache")
     ap.add_argument("--shape", default=None,
-                    help="B,kv_len,Hq,Hkv,D,P[,bf16|fp16|fp8]: a uniform batch of another shape instead of a BASELINE "
+                    help="B,kv_len,Hq,Hkv,D,P[,bf16|fp16|fp8]: a uniform batch of another shape instead of a numbered "
                          "config (secondary measurements: other head dims, groups, batch sizes)")
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: a kernel of known traffic against which "

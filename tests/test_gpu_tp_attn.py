@@ -122,3 +122,65 @@ def test_refusals(fd):
     attn.init_from_weights(w, w, w, torch.zeros(64, 128, dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
         attn.fwd(torch.zeros(1, 2, 64, dtype=torch.bfloat16, device=DEV), None, None, None, 0)
+
+
+@pytest.mark.parametrize("cache_kind", ["dense", "paged_fp8"])
+def test_decode_block_in_a_hip_graph(fd, cache_kind):
+    """The reference's engine captures its decode step in a graph and replays it with static input tensors
+    (models/engine.py:75-105).  The whole block -- projections, norm + rotary + append, split, combine -- is
+    captured once here and replayed while the cache grows; every replay is checked against the same step run
+    eagerly on a twin cache."""
+    gen = torch.Generator().manual_seed(12)
+    B, hidden, Hq, Hkv, D, L, prefill, steps = 20, 256, 8, 2, 128, 256, 150, 4
+    dt = torch.bfloat16
+    mk = lambda *s, sc=0.06: (torch.randn(*s, generator=gen) * sc).to(dt)  # noqa: E731
+    attn = fd.layers.TP_Attn()
+    attn._init_parameters(_HFAttn(mk(Hq * D, hidden), mk(Hkv * D, hidden), mk(Hkv * D, hidden), mk(hidden, Hq * D, sc=0.03),
+                                  (1 + mk(D, sc=0.1)).to(dt), (1 + mk(D, sc=0.1)).to(dt)))
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    tab = fd.layers._set_cos_sin_cache(inv_freq.to(DEV), L)
+
+    def new_cache():
+        if cache_kind == "dense":
+            return fd.layers.KV_Cache(num_layers=1, batch_size=B, max_length=L, kv_heads=Hkv, head_dim=D, dtype=dt,
+                                      world_size=1)
+        return fd.layers.PagedKV_Cache(num_layers=1, batch_size=B, max_length=L, kv_heads=Hkv, head_dim=D, dtype=dt,
+                                       page_size=16, fp8=True, seed=1)
+    caches = [new_cache(), new_cache()]
+    start = torch.randint(1, prefill, (B,), generator=gen, dtype=torch.int32)     # ragged: the append also schedules
+    pk, pv = mk(B, prefill, Hkv, D, sc=1.0), mk(B, prefill, Hkv, D, sc=1.0)
+    for c in caches:
+        kc, vc, off = c.update_kv_cache(None, None, 0)
+        bt = c.block_table if c.block_table is not None else torch.arange(B, dtype=torch.int32, device=DEV).view(B, 1)
+        fd.rope_kv_append(pk.to(DEV), pv.to(DEV), kc, vc, bt, off, k_scale=c.k_scale, v_scale=c.v_scale)
+        c.kv_offset.copy_(start)       # only the first start[b] prompt tokens count
+
+    x = torch.zeros(B, 1, hidden, dtype=dt, device=DEV)
+    pos = torch.zeros(B, 1, dtype=torch.long, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        attn.fwd(x, pos, tab, caches[0], 0)         # warm-up outside the capture (library handles, allocator)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    caches[0].kv_offset.copy_(start)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_graph = attn.fwd(x, pos, tab, caches[0], 0)
+    caches[0].kv_offset.copy_(start)
+    # the capture ran no kernel, but the warm-up wrote one token at position start[b]: the replays overwrite it
+
+    for step in range(steps):
+        x.copy_(torch.randn(B, 1, hidden, generator=gen).to(dt))
+        pos.copy_(caches[0].get_kv_len()[:, None].long())
+        graph.replay()
+        caches[0].inc_offset()
+        torch.cuda.synchronize()
+        got = y_graph.clone()
+        y_eager = attn.fwd(x, pos, tab, caches[1], 0)          # eager twin, its own cache
+        caches[1].inc_offset()
+        torch.cuda.synchronize()
+        assert torch.equal(got, y_eager), f"replay {step} differs from the eager step"
+        assert torch.equal(caches[0].k_cache.view(torch.uint8), caches[1].k_cache.view(torch.uint8))
+        assert torch.equal(caches[0].kv_offset, caches[1].kv_offset)
+    assert torch.isfinite(y_eager.float()).all() and float(y_eager.float().abs().max()) > 0
