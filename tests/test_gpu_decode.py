@@ -386,10 +386,41 @@ def test_fp8_dequant_table_through_the_kernel(fd):
 
 
 @pytest.mark.parametrize("num_heads", [(64, 8), (16, 4), (8, 8)])
-def test_fp8_decode_matches_oracle_on_dequantised_cache(fd, num_heads):
-    wl = fd.utils.make_paged_workload("fp8", [1000, 17, 4097], num_heads[0], num_heads[1], 128, 16, torch.bfloat16, 16,
-                                      seed=61, fp8_kv=True)
+@pytest.mark.parametrize("D", [128, 256, 64])
+def test_fp8_decode_matches_oracle_on_dequantised_cache(fd, num_heads, D):
+    wl = fd.utils.make_paged_workload("fp8", [1000, 17, 4097, 0, 33], num_heads[0], num_heads[1], D, 16, torch.bfloat16,
+                                      16, seed=61, fp8_kv=True)
     out, lse = run_decode(fd, wl)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    assert_lse_close(lse, ref_lse)
+    if D != 64:   # head_dim 128 / 256 have an MFMA and a VALU kernel: force each
+        for path, extra in (("valu", {}), ("mfma", dict(waves_per_block=4, plan_splits=False))):
+            out_p, lse_p = run_decode(fd, wl, path=path, **extra)
+            assert_out_close(out_p, ref)
+            assert_lse_close(lse_p, ref_lse)
+
+
+def test_fp8_d256_dequant_table_and_soft_cap(fd):
+    """All byte patterns through the head_dim-256 fp8 kernel (kv_len == 1: out == dequantised V[0], exact),
+    then a soft-capped, fp16-query run against the oracle."""
+    tab = torch.from_numpy(oracle.fp8_e4m3fn_decode_table())
+    bytes_ = torch.arange(256, dtype=torch.uint8)
+    bytes_[0x7f] = 0
+    bytes_[0xff] = 0x80
+    v = bytes_.view(1, 1, 1, 256).clone()
+    k = torch.full_like(v, 0x38)
+    q = torch.ones(1, 4, 256, dtype=torch.bfloat16)
+    out = fd.gqa_fwd_batch_decode(q.to(DEV), k.to(DEV), v.to(DEV), None, [1], torch.tensor([1], dtype=torch.int32, device=DEV),
+                                  torch.zeros(1, 1, dtype=torch.int32, device=DEV), 0.0625,
+                                  output_combine=torch.empty(1, 4, 256, dtype=torch.float32, device=DEV),
+                                  k_scale=torch.tensor([0.5], device=DEV), v_scale=torch.tensor([3.0], device=DEV), path="mfma")
+    torch.cuda.synchronize()
+    for h in range(4):
+        assert torch.equal(out[0, h].cpu(), tab[v[0, 0, 0].long()] * 3.0)
+    wl = fd.utils.make_paged_workload("fp8_d256_cap", [700, 129, 31], 24, 2, 256, 1, torch.float16, 32, seed=62,
+                                      soft_cap=30.0, fp8_kv=True)
+    out, lse = run_decode(fd, wl, path="mfma")
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)

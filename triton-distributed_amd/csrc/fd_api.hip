@@ -42,13 +42,13 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
   *shift = k;
 }
 
-// Shapes the MFMA split kernels are built for: head_dim 128 with a 16-bit or fp8-e4m3 cache, head_dim 64 or 256 with
+// Shapes the MFMA split kernels are built for: head_dim 128 or 256 with a 16-bit or fp8-e4m3 cache, head_dim 64 with
 // a 16-bit cache; any GQA group (blocks of 16 query heads, the last one padded: even with one
 // query head per KV head the MFMA kernels stream faster than the VALU kernel, 46.1 vs 50.2 us on config 2's shape as MHA,
 // 46.1 vs 78.9 us with 3 query heads per KV head).
 bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
   const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
-  const bool dim_ok = (head_dim == 128 && (kv16 || kv_dtype == FD_FP8_E4M3)) || ((head_dim == 64 || head_dim == 256) && kv16);
+  const bool dim_ok = ((head_dim == 128 || head_dim == 256) && (kv16 || kv_dtype == FD_FP8_E4M3)) || (head_dim == 64 && kv16);
   (void)group;
   return dim_ok;
 }
@@ -176,7 +176,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs head_dim 128 (or 64 / 256 with a 16-bit cache), a 16-bit query with a KV cache "
+                "%s: MFMA path needs head_dim 128 / 256 (or 64 with a 16-bit cache), a 16-bit query with a KV cache "
                 "of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
@@ -186,7 +186,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (use_mfma) {
     a.hbsz = G < 16 ? G : 16;
     a.nhb = (G + 15) / 16;
-    tile = (kv_fp8 || D == 64) ? 64 : (D == 256 ? 16 : 32);
+    tile = kv_fp8 ? (D == 256 ? 32 : 64) : (D == 64 ? 64 : (D == 256 ? 16 : 32));
   } else {
     a.hbsz = G >= 3 ? 4 : G;
     a.nhb = (G + a.hbsz - 1) / a.hbsz;
@@ -215,7 +215,9 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   }
 
   int rc;
-  if (use_mfma && kv_fp8) {
+  if (use_mfma && kv_fp8 && D == 256) {
+    rc = fd_launch_split_mfma_fp8_d256((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
+  } else if (use_mfma && kv_fp8) {
     rc = fd_launch_split_mfma_fp8((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
   } else if (use_mfma && D == 64) {
     rc = fd_launch_split_mfma_d64((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);

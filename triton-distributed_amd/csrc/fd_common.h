@@ -384,6 +384,7 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap);
 int fd_launch_split_mfma_d64(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap);
 int fd_launch_split_mfma_d256(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap);
+int fd_launch_split_mfma_fp8_d256(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap);
 int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap);
 int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int waves);
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a);

@@ -2,7 +2,7 @@
 //
 // Replaces kernel_gqa_fwd_batch_decode_split_kv
 // (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) where the MFMA
-// kernels do not apply: fp32 caches or queries, fp8 caches with head_dim 64 / 256,
+// kernels do not apply: fp32 caches or queries, fp8 caches with head_dim 64,
 // a cache dtype that differs from the query's -- and whenever the caller forces
 // this path.
 // Any KV dtype (fp32, fp16, bf16, fp8-e4m3 with per-head scales) is dequantised
