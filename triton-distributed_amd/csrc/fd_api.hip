@@ -200,6 +200,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
   if (use_mfma && !fuse) a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs);
+  a.nsub = waves;
   waves *= a.hpw;   // total waves of a workgroup
 
   // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS

@@ -43,6 +43,7 @@ struct SplitArgs {
   int32_t nhb;      // head blocks per KV head
   int32_t hbsz;     // query heads per head block
   int32_t hpw;      // adjacent KV heads per workgroup (one wave each; x token sub-ranges = waves)
+  int32_t nsub;     // token sub-ranges of a split (waves per KV head); the workgroup has hpw * nsub waves
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
@@ -158,6 +159,23 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Fetches everything a wave needs before its first K/V request from the kernel-argument segment NOW, as one
+// batch of scalar loads.  Left to itself the compiler loads each field right before its first use, which puts
+// half a dozen dependent scalar-load round trips in front of the first table lookup; a value pinned in an SGPR
+// here has to be loaded here (input-only constraints: the values themselves, and what the compiler knows about the
+// pointers, stay as they are).
+__device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
+#define FD_PIN(f) asm volatile("" ::"s"(a.f))
+  FD_PIN(q); FD_PIN(k); FD_PIN(v); FD_PIN(bt); FD_PIN(kv_lens); FD_PIN(order); FD_PIN(order_lens);
+  FD_PIN(sq_b); FD_PIN(sq_h); FD_PIN(sk_t); FD_PIN(sk_h); FD_PIN(sv_t); FD_PIN(sv_h); FD_PIN(sbt);
+  FD_PIN(sm_scale); FD_PIN(batch); FD_PIN(G); FD_PIN(S); FD_PIN(P); FD_PIN(max_pages); FD_PIN(num_pages);
+  FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(s_magic); FD_PIN(s_shift);
+  // what the epilogue reads, so that it does not wait for the argument segment either
+  FD_PIN(out); FD_PIN(lse); FD_PIN(so_b); FD_PIN(so_h); FD_PIN(so_s); FD_PIN(tickets); FD_PIN(mid_dtype);
+  FD_PIN(vec_out); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
+#undef FD_PIN
+}
+
 // Work item of a wave: grid = ((Hkv / hpw) * nhb, S, batch).  A workgroup owns hpw ADJACENT KV heads of
 // one (sequence, split): wave w works on head kvh0 + w % hpw and on token sub-range w / hpw of the
 // split.  Sibling waves therefore request neighbouring 128/256-byte pieces of the same token rows
@@ -173,6 +191,14 @@ struct WorkItem {
 
 __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   WorkItem w;
+  // The sequence and its length first: these scalar loads head the chain length -> block table -> K/V rows that
+  // every wave has to walk before it can stream.
+  const int r = blockIdx.z;
+  int b = a.order ? a.order[r] : r;
+  w.b = min(max(b, 0), a.batch - 1);
+  int64_t len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
+  fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
+
   const int wave = threadIdx.x >> 6;
   int grp;
   if (a.nhb == 1) {
@@ -186,19 +212,15 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     w.kvh0 = grp;
     w.kvh = grp;
     w.sub = wave;
-    w.nsub = blockDim.x >> 6;
+    w.nsub = a.nsub;
   } else {
     w.kvh0 = grp * a.hpw;
     w.sub = wave / a.hpw;
     w.kvh = w.kvh0 + (wave - w.sub * a.hpw);
-    w.nsub = (blockDim.x >> 6) / a.hpw;
+    w.nsub = a.nsub;
   }
   w.s = blockIdx.y;
-  const int r = blockIdx.z;
-  int b = a.order ? a.order[r] : r;
-  w.b = min(max(b, 0), a.batch - 1);
   int64_t cap = (int64_t)a.max_pages * a.P;
-  int64_t len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
   // per = ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)
@@ -236,7 +258,7 @@ template <int HB, int D>
 __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float* part, int stride,
                                                 const WorkItem& w, int nheads, bool scale_by_v) {
   const int tid = threadIdx.x;
-  const int nthreads = blockDim.x;
+  const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
   constexpr int D4 = D / 4;
   const int per_head = nheads * D4;
   for (int e = tid; e < a.hpw * per_head; e += nthreads) {
@@ -297,7 +319,7 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
                                               float* s_lse) {
   __shared__ int s_last;
   const int tid = threadIdx.x;
-  const int nth = blockDim.x;
+  const int nth = 64 * a.hpw * a.nsub;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // vmcnt(0): the write-through stores have completed
   __syncthreads();
   if (tid == 0) {
