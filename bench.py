@@ -141,6 +141,46 @@ def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step, pools, kv
     }
 
 
+def measure_decode_block(torch, fd, wl, dev, steps, warmup):
+    """The caller of the path: one attention block at decode time (QKV projection, rotary + append, split-KV
+    decode, combine, output projection) for a model whose hidden size is Hq * D, on a paged cache holding this
+    workload's lengths -- launched eagerly from Python, and replayed from a HIP graph as a serving loop would."""
+    B, Hq, D = wl.q.shape
+    _, P, Hkv, _ = wl.k_cache.shape
+    if wl.q.dtype not in (torch.bfloat16, torch.float16):
+        return None
+    hidden = Hq * D
+    dt = wl.q.dtype
+    fp8 = wl.k_scale is not None
+    max_len = -(-(int(wl.kv_lens.max()) + 64) // P) * P
+    attn = fd.layers.TP_Attn()
+    w = lambda *shape: (torch.randn(*shape, device=dev) * 0.02).to(dt)  # noqa: E731
+    attn.init_from_weights(w(Hq * D, hidden), w(Hkv * D, hidden), w(Hkv * D, hidden), w(hidden, Hq * D), head_dim=D)
+    cache = fd.layers.PagedKV_Cache(num_layers=1, batch_size=B, max_length=max_len, kv_heads=Hkv, head_dim=D, dtype=dt,
+                                    page_size=P, fp8=fp8)
+    cache.kv_offset.copy_(wl.kv_lens)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32, device=dev) / D))
+    tab = fd.layers._set_cos_sin_cache(inv_freq, max_len)
+    x = torch.randn(B, 1, hidden, device=dev).to(dt)
+    pos = wl.kv_lens[:, None].long()
+
+    def eager(_):
+        attn.fwd(x, pos, tab, cache, 0)
+    t_eager = _time_us(torch, eager, steps, warmup)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eager(0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        attn.fwd(x, pos, tab, cache, 0)
+    t_graph = _time_us(torch, lambda _: graph.replay(), steps, warmup)
+    return {"hidden_size": hidden, "launches": "2 GEMMs (hipBLASLt) + norm/rotary/append + split-KV decode (+ combine)",
+            "eager_us": round(t_eager, 3), "hip_graph_us": round(t_graph, 3)}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -324,6 +364,9 @@ def main():
 
     if not args.no_write_side:
         result["write_side"] = measure_write_side(torch, fd, wl, dev, args.steps, args.warmup, step, pools, S)
+        block = measure_decode_block(torch, fd, wl, dev, args.steps, args.warmup)
+        if block is not None:
+            result["decode_block"] = block
 
     if not args.no_cpu_baseline:
         import oracle  # the checker, timed as the CPU baseline only
