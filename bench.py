@@ -390,11 +390,14 @@ def main():
         sub_lens = [lens[i] for i in rows]
         times = []
         ref = ref_lse = None
-        for it in range(4):  # 1 warm-up + 3 timed
+        t_begin = time.perf_counter()
+        it = 0
+        while it < 4 or (time.perf_counter() - t_begin < 10.0 and it < 60):  # 1 warm-up, then >= 3 runs / about 10 s
             t = time.perf_counter()
             ref, ref_lse = oracle.ref_paged_attn_lse(qc, kc, vc, sub_lens, bt, wl_cpu.scale, soft_cap=wl_cpu.soft_cap)
             if it:
                 times.append(time.perf_counter() - t)
+            it += 1
         frac_tokens = sum(sub_lens) / max(1, sum(lens))
         cpu_us = statistics.median(times) * 1e6 / frac_tokens
         if wl_cpu.extra_out is None:
@@ -405,7 +408,8 @@ def main():
         result["cpu_baseline"] = {
             "value": round(cpu_us, 1), "unit": "us/decode step", "cores": torch_threads, "kind": "port",
             "sample": f"oracle.ref_paged_attn_lse (fp32 PyTorch restatement of the reference's ref_paged_attn) on "
-                      f"sequences 0..{n_seq - 1} of {B} of the same seeded workload, median of 3 runs, scaled by "
+                      f"sequences 0..{n_seq - 1} of {B} of the same seeded workload, median of {len(times)} runs "
+                      f"({sum(times):.1f} s of CPU work), scaled by "
                       f"1/{frac_tokens:.4f} (token share) to the whole step; host cpu_count={os.cpu_count()}",
         }
     print(json.dumps(result))
