@@ -14,16 +14,19 @@ struct Fp8 {};   // tag: OCP e4m3fn bit patterns, one byte each
 template <typename T> struct ElemBytes { static constexpr int v = sizeof(T); };
 template <> struct ElemBytes<Fp8> { static constexpr int v = 1; };
 
-template <typename T>
+// STREAM: the data is read once (activations) -- non-temporal; otherwise (norm weights, shared by every row) cached.
+template <typename T, bool STREAM = true>
 __device__ __forceinline__ void load8(const void* base, int64_t idx, float* x) {
   if constexpr (sizeof(T) == 4) {
     const f32x4* p = (const f32x4*)((const float*)base + idx);
-    const f32x4 a = p[0], b = p[1];
+    const f32x4 a = STREAM ? __builtin_nontemporal_load(p) : p[0];
+    const f32x4 b = STREAM ? __builtin_nontemporal_load(p + 1) : p[1];
 #pragma unroll
     for (int i = 0; i < 4; ++i) { x[i] = a[i]; x[4 + i] = b[i]; }
   } else {
     typedef T vec8 __attribute__((ext_vector_type(8)));
-    const vec8 v = *(const vec8*)((const T*)base + idx);
+    const vec8* p = (const vec8*)((const T*)base + idx);
+    const vec8 v = STREAM ? __builtin_nontemporal_load(p) : *p;
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] = (float)v[i];
   }
@@ -52,13 +55,14 @@ __device__ __forceinline__ void store8(void* base, int64_t idx, const float* x, 
     f32x4 a, b;
 #pragma unroll
     for (int i = 0; i < 4; ++i) { a[i] = x[i]; b[i] = x[4 + i]; }
-    p[0] = a; p[1] = b;
+    __builtin_nontemporal_store(a, p);
+    __builtin_nontemporal_store(b, p + 1);
   } else if constexpr (sizeof(T) == 2) {
     typedef T vec8 __attribute__((ext_vector_type(8)));
     vec8 v;
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (T)x[i];
-    *(vec8*)((T*)base + idx) = v;
+    __builtin_nontemporal_store(v, (vec8*)((T*)base + idx));
   } else {
     u32x2 w;
     uint32_t lo = 0, hi = 0;
@@ -67,7 +71,7 @@ __device__ __forceinline__ void store8(void* base, int64_t idx, const float* x, 
     hi = quant2_fp8(x[4], x[5], scale, hi, false);
     hi = quant2_fp8(x[6], x[7], scale, hi, true);
     w[0] = lo; w[1] = hi;
-    *(u32x2*)((uint8_t*)base + idx) = w;
+    __builtin_nontemporal_store(w, (u32x2*)((uint8_t*)base + idx));
   }
 }
 
@@ -102,8 +106,8 @@ __device__ __forceinline__ void rms_norm_row(float* x1, float* x2, const void* w
   for (int off = 1; off < cpr; off <<= 1) ss += __shfl_xor(ss, off);   // the row's lanes are aligned to cpr
   const float rstd = 1.0f / sqrtf(ss / (float)(2 * half) + eps);
   float w1[8], w2[8];
-  load8<SRC>(w, e0, w1);
-  load8<SRC>(w, half + e0, w2);
+  load8<SRC, false>(w, e0, w1);
+  load8<SRC, false>(w, half + e0, w2);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     x1[i] = round_through<SRC>(x1[i] * rstd * w1[i]);
