@@ -1,0 +1,58 @@
+"""Seeded random sweep over shapes and launch options of the decode path against the CPU oracle: every MFMA and
+VALU kernel, tile boundaries (kv_len around multiples of 16 / 32 / 64), more waves than tiles, empty sequences,
+sibling-head workgroups, caller-visible and internal partials, the scheduler and the fused combine."""
+import random
+
+import pytest
+import torch
+
+from helpers import assert_lse_close, assert_out_close, oracle_decode, run_decode
+
+pytestmark = pytest.mark.gpu
+
+CASES = 160
+
+
+def _case(i):
+    rng = random.Random(9000 + i)
+    D = rng.choice([64, 128, 128, 256])
+    kind = rng.choice(["bf16", "fp16", "fp8", "fp32"]) if D != 64 else rng.choice(["bf16", "fp16", "fp32"])
+    Hkv = rng.choice([1, 2, 4, 8])
+    G = rng.choice([1, 2, 3, 4, 6, 8, 16, 20])
+    P = rng.choice([1, 4, 16, 16, 32, 128])
+    B = rng.choice([1, 2, 3, 5, 9])
+    edge = [0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 257, 511, 513]
+    lens = [rng.choice(edge) if rng.random() < 0.6 else rng.randint(1, 1500) for _ in range(B)]
+    if max(lens) == 0:
+        lens[0] = 40
+    return dict(D=D, kind=kind, Hq=Hkv * G, Hkv=Hkv, P=P, lens=lens, kv_split=rng.choice([1, 2, 5, 8, 32]),
+                soft_cap=rng.choice([0.0, 0.0, 30.0]), waves=rng.choice([0, 0, 1, 2, 4, 8]),
+                variant=rng.choice(["plain", "plain", "persistent", "intra"]), fuse=rng.random() < 0.2,
+                plan=rng.random() < 0.5, path=rng.choice(["auto", "auto", "valu"]))
+
+
+@pytest.mark.parametrize("i", range(CASES))
+def test_random_shape(fd, i):
+    c = _case(i)
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp8": torch.bfloat16, "fp32": torch.float32}[c["kind"]]
+    wl = fd.utils.make_paged_workload(f"rand{i}", c["lens"], c["Hq"], c["Hkv"], c["D"], c["P"], dtype, c["kv_split"],
+                                      seed=7000 + i, soft_cap=c["soft_cap"], fp8_kv=c["kind"] == "fp8", pool_slack_pages=3)
+    kw = dict(path=c["path"], waves_per_block=c["waves"], plan_splits=c["plan"])
+    if c["variant"] != "intra":
+        kw["fuse_combine"] = c["fuse"]
+    ref, ref_lse = oracle_decode(wl)
+    fp32 = dtype == torch.float32
+    if c["variant"] == "intra":
+        g = wl.to("cuda:0")
+        if g.k_scale is not None:
+            kw.update(k_scale=g.k_scale, v_scale=g.v_scale)
+        res = fd.gqa_fwd_batch_decode_intra_rank(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
+                                                 g.soft_cap, kv_split=g.kv_split, **kw)
+        torch.cuda.synchronize()
+        out, lse = res[..., :c["D"]].cpu(), res[..., c["D"]].float().cpu()
+        lse_rtol = 1e-5 if fp32 else 1e-2      # the LSE column has the output's dtype
+    else:
+        out, lse = run_decode(fd, wl, variant=c["variant"], **kw)
+        lse_rtol = 1e-5 if fp32 else 1e-3
+    assert_out_close(out, ref, atol=2e-4 if fp32 else 2e-2)
+    assert_lse_close(lse, ref_lse, rtol=lse_rtol)
