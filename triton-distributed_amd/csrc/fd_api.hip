@@ -370,13 +370,13 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
                  int32_t batch, int32_t new_tokens, int64_t stride_kn_b, int64_t stride_kn_t, int64_t stride_kn_h,
                  int64_t stride_vn_b, int64_t stride_vn_t, int64_t stride_vn_h, int64_t stride_k_tok,
                  int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_table_bs,
-                 const fd_qk_prep* rope, const fd_params* p) {
+                 const fd_qk_prep* prep, const fd_params* p) {
   const char* fn = "fd_kv_append";
   if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (batch < 0 || new_tokens < 0) return fail(FD_ERR_INVALID_ARG, "%s: batch %d, new_tokens %d", fn, batch, new_tokens);
   if (batch == 0 || new_tokens == 0) return FD_OK;
   const bool append = k_new || v_new;
-  const bool with_q = rope && rope->q;
+  const bool with_q = prep && prep->q;
   if (seq_order_out && !append) return fail(FD_ERR_INVALID_ARG, "%s: seq_order_out needs k_new / v_new and kv_lens", fn);
   if (seq_order_out && batch > 4096)
     return fail(FD_ERR_TOO_LARGE, "%s: seq_order_out with batch %d > 4096 (use fd_schedule)", fn, batch);
@@ -425,35 +425,35 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
     a.sk_t = stride_k_tok; a.sk_h = stride_k_h; a.sv_t = stride_v_tok; a.sv_h = stride_v_h;
     a.sbt = stride_table_bs; a.P = p->page_size; a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
   }
-  if (rope) {
-    if (!rope->cos_sin && !rope->q_norm_weight && !rope->k_norm_weight)
+  if (prep) {
+    if (!prep->cos_sin && !prep->q_norm_weight && !prep->k_norm_weight)
       return fail(FD_ERR_INVALID_ARG, "%s: prep without cos_sin and without a norm weight", fn);
-    if (rope->cos_sin) {
-      if (!rope->position_ids) return fail(FD_ERR_INVALID_ARG, "%s: cos_sin needs position_ids", fn);
-      if (rope->max_positions <= 0) return fail(FD_ERR_INVALID_ARG, "%s: prep->max_positions %d", fn, rope->max_positions);
-      if (rope->position_dtype != 0 && rope->position_dtype != 1)
-        return fail(FD_ERR_INVALID_ARG, "%s: prep->position_dtype %d (0: int32, 1: int64)", fn, rope->position_dtype);
-      if (!aligned16(rope->cos_sin) || rope->stride_cos_sin % 4 || rope->stride_cos_sin < D)
+    if (prep->cos_sin) {
+      if (!prep->position_ids) return fail(FD_ERR_INVALID_ARG, "%s: cos_sin needs position_ids", fn);
+      if (prep->max_positions <= 0) return fail(FD_ERR_INVALID_ARG, "%s: prep->max_positions %d", fn, prep->max_positions);
+      if (prep->position_dtype != 0 && prep->position_dtype != 1)
+        return fail(FD_ERR_INVALID_ARG, "%s: prep->position_dtype %d (0: int32, 1: int64)", fn, prep->position_dtype);
+      if (!aligned16(prep->cos_sin) || prep->stride_cos_sin % 4 || prep->stride_cos_sin < D)
         return fail(FD_ERR_ALIGNMENT, "%s: cos_sin rows must hold head_dim floats and be 16-byte aligned", fn);
-      a.cos_sin = rope->cos_sin; a.s_cs = rope->stride_cos_sin; a.pos = rope->position_ids;
-      a.pos_i64 = rope->position_dtype; a.max_pos = rope->max_positions;
-      a.sp_b = rope->stride_pos_b; a.sp_t = rope->stride_pos_t;
+      a.cos_sin = prep->cos_sin; a.s_cs = prep->stride_cos_sin; a.pos = prep->position_ids;
+      a.pos_i64 = prep->position_dtype; a.max_pos = prep->max_positions;
+      a.sp_b = prep->stride_pos_b; a.sp_t = prep->stride_pos_t;
     }
-    if (!aligned16(rope->q_norm_weight) || !aligned16(rope->k_norm_weight))
+    if (!aligned16(prep->q_norm_weight) || !aligned16(prep->k_norm_weight))
       return fail(FD_ERR_ALIGNMENT, "%s: norm weights must be 16-byte aligned", fn);
-    if (rope->q_norm_weight && !with_q) return fail(FD_ERR_INVALID_ARG, "%s: q_norm_weight without prep->q", fn);
-    if (rope->k_norm_weight && !append) return fail(FD_ERR_INVALID_ARG, "%s: k_norm_weight without k_new", fn);
-    a.qn_w = rope->q_norm_weight; a.kn_w = rope->k_norm_weight;
-    a.qn_eps = rope->q_norm_eps; a.kn_eps = rope->k_norm_eps;
+    if (prep->q_norm_weight && !with_q) return fail(FD_ERR_INVALID_ARG, "%s: q_norm_weight without prep->q", fn);
+    if (prep->k_norm_weight && !append) return fail(FD_ERR_INVALID_ARG, "%s: k_norm_weight without k_new", fn);
+    a.qn_w = prep->q_norm_weight; a.kn_w = prep->k_norm_weight;
+    a.qn_eps = prep->q_norm_eps; a.kn_eps = prep->k_norm_eps;
     if (with_q) {
-      if (!rope->q_out) return fail(FD_ERR_INVALID_ARG, "%s: prep->q without prep->q_out", fn);
-      if (!aligned16(rope->q) || !aligned16(rope->q_out) || rope->stride_q_b % src16 || rope->stride_q_t % src16 ||
-          rope->stride_q_h % src16 || rope->stride_qo_b % src16 || rope->stride_qo_t % src16 ||
-          rope->stride_qo_h % src16)
+      if (!prep->q_out) return fail(FD_ERR_INVALID_ARG, "%s: prep->q without prep->q_out", fn);
+      if (!aligned16(prep->q) || !aligned16(prep->q_out) || prep->stride_q_b % src16 || prep->stride_q_t % src16 ||
+          prep->stride_q_h % src16 || prep->stride_qo_b % src16 || prep->stride_qo_t % src16 ||
+          prep->stride_qo_h % src16)
         return fail(FD_ERR_ALIGNMENT, "%s: q / q_out rows must be 16-byte aligned (pointer and strides)", fn);
-      a.q = rope->q; a.q_out = rope->q_out;
-      a.sq_b = rope->stride_q_b; a.sq_t = rope->stride_q_t; a.sq_h = rope->stride_q_h;
-      a.sqo_b = rope->stride_qo_b; a.sqo_t = rope->stride_qo_t; a.sqo_h = rope->stride_qo_h;
+      a.q = prep->q; a.q_out = prep->q_out;
+      a.sq_b = prep->stride_q_b; a.sq_t = prep->stride_q_t; a.sq_h = prep->stride_q_h;
+      a.sqo_b = prep->stride_qo_b; a.sqo_t = prep->stride_qo_t; a.sqo_h = prep->stride_qo_h;
     }
   }
   int rc = fd_launch_kv_append((hipStream_t)stream, a, p->q_dtype, kv_dtype);

@@ -23,6 +23,10 @@ from .._lib import FdParams, FdQkPrep, check, fd_dtype_of, load_library, stream_
 from .flash_decode import _decode, _require_cuda
 
 
+def _ptr(t: Optional[torch.Tensor]):
+    return t.data_ptr() if t is not None else None
+
+
 def _prep_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdQkPrep:
     r = FdQkPrep()
     if cos_sin is None:
@@ -54,12 +58,12 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
     With ``cos_sin`` (fp32 ``[max_pos, D]``) and ``position_ids`` (``[B, T]`` int32/int64) K is rotated before it
     is stored and ``q`` ``[B, T, Hq, D]`` (if given) is rotated into ``q_out`` (default: a new tensor; may be
     ``q``) in the same launch.  ``q_norm`` / ``k_norm`` = ``(weight [D], eps)`` apply the per-head RMS norm of the
-    reference's block (tp_attn.py:252-258) to q / k before the rotation.  A uint8 / float8_e4m3fn cache with ``k_scale`` / ``v_scale`` ``[Hkv]`` stores
-    ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out`` (int32 ``[B]``, not ``kv_lens``) receives
-    the grown lengths; ``seq_order_out`` (int32 ``[2, B]``, ``B <= 4096``) the longest-first issue order for the
-    decode that follows (row 0: what ``schedule_sequences`` would compute, without a launch of its own) and the
-    grown lengths in that order (row 1: the decode's ``seq_order_lens``).  Returns
-    ``q_out`` (or ``None`` without ``q``).
+    reference's block (tp_attn.py:252-258) to q / k before the rotation.  A uint8 / float8_e4m3fn cache with
+    ``k_scale`` / ``v_scale`` ``[Hkv]`` stores ``clamp(x / scale, +-448)`` rounded to e4m3fn.  ``kv_lens_out``
+    (int32 ``[B]``, not ``kv_lens``) receives the grown lengths; ``seq_order_out`` (int32 ``[2, B]``,
+    ``B <= 4096``) the longest-first issue order for the decode that follows (row 0: what ``schedule_sequences``
+    would compute, without a launch of its own) and the grown lengths in that order (row 1: the decode's
+    ``seq_order_lens``).  Returns ``q_out`` (or ``None`` without ``q``).
     """
     lib = load_library()
     append = k_new is not None
@@ -74,7 +78,6 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
     p.q_dtype = fd_dtype_of(src)
     p.q_heads = q.shape[2] if q is not None else 1
     p.kv_heads = k_new.shape[2] if append else 1
-    ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
     skn = svn = (0, 0, 0)
     sk = sv = (0, 0)
     sbt = 0
@@ -97,35 +100,35 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
         p.num_pages = k_cache.shape[0]
         p.max_pages_per_seq = block_table.shape[1]
         p.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
-        p.k_scale, p.v_scale = ptr(k_scale), ptr(v_scale)
+        p.k_scale, p.v_scale = _ptr(k_scale), _ptr(v_scale)
         skn, svn = k_new.stride()[:3], v_new.stride()[:3]
         sk, sv = (k_cache.stride(1), k_cache.stride(2)), (v_cache.stride(1), v_cache.stride(2))
         sbt = block_table.stride(0)
-    rope = None
+    prep = None
     if cos_sin is not None or q_norm is not None or k_norm is not None:
-        rope = _prep_struct(cos_sin, position_ids, head_dim, bsz, seq)
+        prep = _prep_struct(cos_sin, position_ids, head_dim, bsz, seq)
         for name, norm in (("q", q_norm), ("k", k_norm)):
             if norm is not None:
                 w, eps = norm
                 _require_cuda(w)
                 assert w.dtype == src.dtype and w.is_contiguous() and w.numel() == head_dim
-                setattr(rope, name + "_norm_weight", w.data_ptr())
-                setattr(rope, name + "_norm_eps", float(eps))
+                setattr(prep, name + "_norm_weight", w.data_ptr())
+                setattr(prep, name + "_norm_eps", float(eps))
         if q is not None:
             assert q.dim() == 4 and q.shape[0] == bsz and q.shape[1] == seq and q.shape[3] == head_dim
             assert q.dtype == src.dtype and q.stride(-1) == 1
             if q_out is None:
                 q_out = torch.empty_like(q)
             assert q_out.shape == q.shape and q_out.dtype == q.dtype and q_out.stride(-1) == 1
-            rope.q, rope.q_out = q.data_ptr(), q_out.data_ptr()
-            rope.stride_q_b, rope.stride_q_t, rope.stride_q_h = q.stride()[:3]
-            rope.stride_qo_b, rope.stride_qo_t, rope.stride_qo_h = q_out.stride()[:3]
+            prep.q, prep.q_out = q.data_ptr(), q_out.data_ptr()
+            prep.stride_q_b, prep.stride_q_t, prep.stride_q_h = q.stride()[:3]
+            prep.stride_qo_b, prep.stride_qo_t, prep.stride_qo_h = q_out.stride()[:3]
     elif q is not None:
         raise RuntimeError("rope_kv_append: q is only processed together with cos_sin / position_ids or a norm")
     check(lib.fd_kv_append(
-        stream_handle(stream, src.device.index), ptr(k_new), ptr(v_new), ptr(k_cache), ptr(v_cache), ptr(block_table),
-        ptr(kv_lens), ptr(kv_lens_out), ptr(seq_order_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
-        byref(rope) if rope is not None else None, byref(p)))
+        stream_handle(stream, src.device.index), _ptr(k_new), _ptr(v_new), _ptr(k_cache), _ptr(v_cache),
+        _ptr(block_table), _ptr(kv_lens), _ptr(kv_lens_out), _ptr(seq_order_out), bsz, seq, *skn, *svn, *sk, *sv, sbt,
+        byref(prep) if prep is not None else None, byref(p)))
     return q_out if q is not None else None
 
 
