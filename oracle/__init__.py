@@ -5,6 +5,10 @@ Nothing in the shipped package imports this directory.  Only the test-suite,
 import it, and only as the checker -- never as the thing being measured or
 shipped.  The product path raises when its HIP library is missing; it never
 routes through this code.
+
+``oracle/c/ref_decode.c`` is a second, independent restatement of the decode in plain C (built by
+``oracle/c/build.py``); tests/test_c_oracle.py holds the two against each other and the C consumer of the ABI
+under tests/c_abi/ checks the library against it with no Python in the loop.
 """
 from .ref_decode import (  # noqa: F401
     ref_paged_attn,
