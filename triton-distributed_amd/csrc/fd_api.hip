@@ -199,7 +199,22 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
-  if (use_mfma && !fuse) a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs);
+  if (use_mfma && !fuse && a.nhb > 1) {
+    // more than 16 query heads per KV head: the head blocks of a KV head share a workgroup (largest divisor of
+    // nhb that keeps the workgroup at 8 waves and the grid at one workgroup per CU), so that they read their
+    // common K/V rows in step
+    int h = 8 / waves;
+    const char* env = getenv("FD_HEADS_PER_BLOCK");   // same tuning override as for sibling KV heads
+    if (env && atoi(env) > 0 && atoi(env) < h) h = atoi(env);
+    while (h > 1 && (a.nhb % h != 0 || wgs / h < kMinWorkgroups)) --h;
+    if (h > 1) {
+      a.hpw = h;
+      a.member_hb = 1;
+    }
+  } else if (use_mfma && !fuse) {
+    a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs);
+  }
+  a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / a.hpw * a.nhb;
   a.nsub = waves;
   waves *= a.hpw;   // total waves of a workgroup
 

@@ -44,6 +44,9 @@ struct SplitArgs {
   int32_t hbsz;     // query heads per head block
   int32_t hpw;      // adjacent KV heads per workgroup (one wave each; x token sub-ranges = waves)
   int32_t nsub;     // token sub-ranges of a split (waves per KV head); the workgroup has hpw * nsub waves
+  int32_t member_hb;  // 1: the hpw members of a workgroup are head blocks of ONE KV head (groups above 16 query
+                      // heads: the blocks read the same K/V rows in step, so the rows come from HBM once)
+  int32_t grid_x;   // workgroups per (sequence, split)
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
@@ -169,7 +172,8 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
   FD_PIN(q); FD_PIN(k); FD_PIN(v); FD_PIN(bt); FD_PIN(kv_lens); FD_PIN(order); FD_PIN(order_lens);
   FD_PIN(sq_b); FD_PIN(sq_h); FD_PIN(sk_t); FD_PIN(sk_h); FD_PIN(sv_t); FD_PIN(sv_h); FD_PIN(sbt);
   FD_PIN(sm_scale); FD_PIN(batch); FD_PIN(G); FD_PIN(S); FD_PIN(P); FD_PIN(max_pages); FD_PIN(num_pages);
-  FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(s_magic); FD_PIN(s_shift);
+  FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(member_hb); FD_PIN(s_magic);
+  FD_PIN(s_shift);
   // what the epilogue reads, so that it does not wait for the argument segment either
   FD_PIN(out); FD_PIN(lse); FD_PIN(so_b); FD_PIN(so_h); FD_PIN(so_s); FD_PIN(tickets); FD_PIN(mid_dtype);
   FD_PIN(vec_out); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
@@ -185,6 +189,7 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
 struct WorkItem {
   int b, s, kvh, hb, start, end;
   int kvh0;   // first KV head of the workgroup
+  int hb0;    // first head block of the workgroup
   int sub;    // token sub-range index of this wave
   int nsub;   // token sub-ranges (waves per head)
 };
@@ -200,23 +205,36 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
 
   const int wave = threadIdx.x >> 6;
-  int grp;
-  if (a.nhb == 1) {
-    grp = blockIdx.x;
-    w.hb = 0;
-  } else {
-    grp = blockIdx.x / a.nhb;
-    w.hb = blockIdx.x - grp * a.nhb;
-  }
-  if (a.hpw == 1) {
-    w.kvh0 = grp;
-    w.kvh = grp;
-    w.sub = wave;
+  if (a.member_hb) {
+    // workgroup = hpw head blocks of one KV head; blockIdx.x = kv head * (nhb / hpw) + block group
+    const int groups = a.nhb / a.hpw;
+    const int kvh = groups == 1 ? (int)blockIdx.x : (int)blockIdx.x / groups;
+    const int hbg = blockIdx.x - kvh * groups;
+    w.sub = wave / a.hpw;
+    w.hb0 = hbg * a.hpw;
+    w.hb = w.hb0 + (wave - w.sub * a.hpw);
+    w.kvh0 = kvh;
+    w.kvh = kvh;
     w.nsub = a.nsub;
   } else {
-    w.kvh0 = grp * a.hpw;
-    w.sub = wave / a.hpw;
-    w.kvh = w.kvh0 + (wave - w.sub * a.hpw);
+    int grp;
+    if (a.nhb == 1) {
+      grp = blockIdx.x;
+      w.hb = 0;
+    } else {
+      grp = blockIdx.x / a.nhb;
+      w.hb = blockIdx.x - grp * a.nhb;
+    }
+    w.hb0 = w.hb;
+    if (a.hpw == 1) {
+      w.kvh0 = grp;
+      w.kvh = grp;
+      w.sub = wave;
+    } else {
+      w.kvh0 = grp * a.hpw;
+      w.sub = wave / a.hpw;
+      w.kvh = w.kvh0 + (wave - w.sub * a.hpw);
+    }
     w.nsub = a.nsub;
   }
   w.s = blockIdx.y;
@@ -252,21 +270,25 @@ __device__ __forceinline__ int token_row(const SplitArgs& a, const int32_t* bt_r
 //
 // LDS layout of wave v's partial (floats): part[v*stride + h*D + d] = un-normalised accumulator,
 // part[v*stride + HB*D + h] = running max (base-2 domain), part[v*stride + HB*D + HB + h] = running
-// sum.  Wave v = head member (v % hpw) + hpw * token sub-range.  Called by every thread of the
-// workgroup after a __syncthreads().  scale_by_v: multiply by v_scale[kv head] (fp8 caches).
+// sum.  Wave v = member (v % hpw) + hpw * token sub-range; a member is a KV head or, for groups above 16 query
+// heads, a head block of the one KV head.  Called by every thread of the workgroup after a __syncthreads() with
+// nheads = the calling wave's head count.  scale_by_v: multiply by v_scale[kv head] (fp8 caches).
 template <int HB, int D>
 __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float* part, int stride,
                                                 const WorkItem& w, int nheads, bool scale_by_v) {
   const int tid = threadIdx.x;
   const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
   constexpr int D4 = D / 4;
-  const int per_head = nheads * D4;
+  // head blocks as members: the last block of a group may hold fewer heads than the others
+  const int per_head = (a.member_hb ? HB : nheads) * D4;
   for (int e = tid; e < a.hpw * per_head; e += nthreads) {
     const int hm = e / per_head;
     const int r = e - hm * per_head;
     const int h = r / D4;
     const int d = (r - h * D4) * 4;
-    const int kvh = w.kvh0 + hm;
+    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+    const int hb = a.member_hb ? w.hb0 + hm : w.hb;
+    if (h >= a.G - hb * HB) continue;
     float M = -INFINITY;
     for (int p = 0; p < w.nsub; ++p) M = fmaxf(M, part[(hm + a.hpw * p) * stride + HB * D + h]);
     float L = 0.f;
@@ -283,7 +305,7 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
     const float out_scale = scale_by_v ? a.v_scale[kvh] : 1.0f;
     float inv = L > 0.f ? out_scale / L : 0.f;
     o *= inv;
-    const int head = kvh * a.G + w.hb * HB + h;
+    const int head = kvh * a.G + hb * HB + h;
     const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;
     const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
     if (a.tickets) {

@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
 }  // namespace
 
 int fd_launch_split_mfma_d256(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
-  const dim3 grid((unsigned)(a.Hkv / a.hpw * a.nhb), (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
   const unsigned block = 64u * waves;
   size_t lds = (size_t)waves * kWaveLds;
   if (a.tickets) {

@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 
 template <int KV, int D>
 int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
-  const dim3 grid((unsigned)(a.Hkv / a.hpw * a.nhb), (unsigned)a.S, (unsigned)a.batch);  // waves = hpw heads x sub-ranges
+  const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
   const unsigned block = 64u * waves;
   void (*kern)(const SplitArgs) = nullptr;
   int gh = a.hbsz;
