@@ -37,7 +37,8 @@ def parse_args():
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
     ap.add_argument("--fuse", action="store_true", help="fuse the combine into the tail of the split kernel")
-    ap.add_argument("--kv-split", type=int, default=0, help="override the workload's kv_split (experiments)")
+    ap.add_argument("--kv-split", type=int, default=0,
+                    help="override the workload's kv_split (experiments); -1: the library's own choice")
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -228,7 +229,8 @@ def main():
 
     out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
-    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev)
+    # kv_split -1: the library chooses the split count and owns the partials
+    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev) if S > 0 else None
     q_lens = [1] * B
     kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=args.path, waves_per_block=args.waves,
               fuse_combine=args.fuse)
@@ -268,13 +270,20 @@ def main():
     from ctypes import byref
     lib = fd.load_library()
     fk = importlib.import_module("triton-distributed_amd.kernels.flash_decode")
-    p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
+    S_bound = S
+    if S == -1:   # the library's own bound, as in the wrapper
+        capacity = wl.block_table.shape[1] * wl.k_cache.shape[1]
+        S_bound = max(fk.DEFAULT_KV_SPLITS, min(fk.MAX_AUTO_KV_SPLITS, capacity // 1024))
+    p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_bound, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
                         wl.k_scale, wl.v_scale, args.path, args.waves)
-    S_eff = S if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
+    p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials
+    S_eff = S_bound if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
     p.num_splits = S_eff
     n_o = B * Hq * S_eff * D
-    mid = workspace[:n_o].view(B, Hq, S_eff, D)
-    lse_split = workspace[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
+    split_ws = workspace if workspace is not None else torch.empty(B * Hq * S_eff * (D + 1), dtype=torch.float32,
+                                                                     device=dev)
+    mid = split_ws[:n_o].view(B, Hq, S_eff, D)
+    lse_split = split_ws[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
     hstream = torch.cuda.current_stream().cuda_stream
     order_ptr = kw["seq_order"].data_ptr() if args.variant == "persistent" else None
 

@@ -96,6 +96,11 @@ typedef struct fd_params {
   const int32_t* seq_order_lens; /* NULL, or [batch] with seq_order: kv_lens[seq_order[r]]
                                at index r (fd_kv_append writes it), so that a workgroup
                                fetches its sequence and its length in one round trip */
+  int32_t split_align;      /* 0: the reference's split ranges, per = ceil(kv_len / S).
+                               A power of two <= 4096: per is rounded up to a multiple of it,
+                               so that splits start on tile boundaries (trailing splits may be
+                               empty).  The result of a step is the same; the partials are not
+                               the reference's.  fd_combine applies the same rule.          */
 } fd_params;
 
 /*
@@ -212,7 +217,8 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  * prologues and fewer partials for the combine.  Returns min(params->num_splits, the split
  * count that (1) reaches about 1024 waves with two waves per (KV head, split) on the MFMA
  * kernels, or about 2048 with four on the VALU kernel, and (2) keeps every split of a
- * full-length sequence at or below 4096 tokens), or a negative fd_status.
+ * full-length sequence at or below 4096 tokens, rounded up to a power of two and then
+ * down to at most params->num_splits), or a negative fd_status.
  * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
  * params->num_splits splits with the reference's ranges.
  */

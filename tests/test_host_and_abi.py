@@ -185,6 +185,10 @@ def test_split_plan_policy(fd):
     assert plan(8, 8, 8, 32, 512) == 8             # MHA runs on the MFMA kernels too
     assert plan(8, 8, 8, 32, 512, kv=L.FD_F32) == 8  # VALU path (fp32 cache): 2048 waves with 4 waves per (head, split)
     assert plan(2, 8, 8, 32, 512) == 32
+    assert plan(3, 32, 8, 32, 512) == 32           # 22 -> the next power of two
+    assert plan(3, 32, 8, 24, 512) == 16           # ... and down again when the caller allows fewer
+    assert plan(1, 96, 12, 128, 65536, P=1) == 64  # one long sequence, the library's own bound: 43 -> 64
+    assert plan(1, 96, 12, 128, 1 << 20, P=1) == 128
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1
     for args in [(3, 16, 16, 32, 83), (7, 6, 1, 5, 1000), (2, 64, 8, 64, 100000)]:

@@ -50,6 +50,7 @@ class FdParams(Structure):
         ("q_dtype", c_int32), ("kv_dtype", c_int32), ("mid_dtype", c_int32), ("out_dtype", c_int32),
         ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
         ("path", c_int32), ("waves_per_block", c_int32), ("seq_order_lens", c_void_p),
+        ("split_align", c_int32),
     ]
 
 

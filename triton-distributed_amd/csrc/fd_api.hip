@@ -163,6 +163,9 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   a.batch = batch; a.Hq = p->q_heads; a.Hkv = p->kv_heads; a.G = G; a.S = p->num_splits; a.P = p->page_size;
   div_magic((uint32_t)p->page_size, &a.div_magic, &a.div_shift);
   div_magic((uint32_t)p->num_splits, &a.s_magic, &a.s_shift);
+  if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
+    return fail(FD_ERR_INVALID_ARG, "%s: split_align %d (0 or a power of two <= 4096)", fn, p->split_align);
+  a.per_mask = p->split_align ? p->split_align - 1 : 0;
   a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
   a.q_dtype = p->q_dtype; a.mid_dtype = p->mid_dtype;
   a.vec_out = (p->mid_dtype == FD_F32 && aligned16(out_split) && stride_o_bs % 4 == 0 && stride_o_h % 4 == 0 &&
@@ -330,7 +333,12 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   // (2) ... and enough that no split of a full-length sequence is longer than kMaxTokensPerSplit
   int64_t s_bal = (max_tokens + kMaxTokensPerSplit - 1) / kMaxTokensPerSplit;
   int64_t s = s_fill > s_bal ? s_fill : s_bal;
-  if (s > p->num_splits) s = p->num_splits;
+  // (3) a power of two: with sequence lengths that are powers of two (or multiples of large ones) every split then
+  // starts on a tile boundary and the waves of a workgroup get equal runs
+  int64_t pow2 = 1;
+  while (pow2 < s) pow2 <<= 1;
+  s = pow2;
+  while (s > p->num_splits) s >>= 1;
   if (s < 1) s = 1;
   return (int)s;
 }
@@ -366,6 +374,9 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   a.vec_mid = (p->mid_dtype == FD_F32 && aligned16(mid_o) && stride_mid_ob % 4 == 0 && stride_mid_oh % 4 == 0 &&
                stride_mid_os % 4 == 0) ? 1 : 0;
   a.all_slots_written = all_slots_written ? 1 : 0;
+  if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
+    return fail(FD_ERR_INVALID_ARG, "fd_combine: split_align %d (0 or a power of two <= 4096)", p->split_align);
+  a.per_mask = p->split_align ? p->split_align - 1 : 0;
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;

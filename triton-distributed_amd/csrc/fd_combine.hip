@@ -41,7 +41,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   int kv_len = 0, per = 0;
   if (a.mode != FD_COMBINE_RANK && !own) {
     kv_len = max(a.seqlens[b], 0);
-    per = (kv_len + S - 1) / S;
+    per = ((kv_len + S - 1) / S + a.per_mask) & ~a.per_mask;
   }
   // LSE of partial s, -inf when the partial is not valid
   auto partial_lse = [&](int s) -> float {

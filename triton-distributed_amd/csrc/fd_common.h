@@ -50,6 +50,7 @@ struct SplitArgs {
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
+  int32_t per_mask;               // split_align - 1 (0: the reference's ranges): tokens per split are rounded up
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
   int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
@@ -72,6 +73,7 @@ struct CombineArgs {
   int64_t s_mb, s_mh, s_ms, s_ob, s_oh;
   int32_t batch, Hq, D, num_partials, num_extra, mode, mid_dtype, out_dtype;
   int32_t vec_mid;  // 1: every mid_o row start is 16-byte aligned (128-bit loads allowed)
+  int32_t per_mask;           // as SplitArgs::per_mask, for the validity of split ranges
   int32_t all_slots_written;  // 1: the partials come from this library's split kernel in the same call, which
                               // writes every slot (empty splits as out = 0, lse = -inf)
 };
@@ -173,7 +175,7 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
   FD_PIN(sq_b); FD_PIN(sq_h); FD_PIN(sk_t); FD_PIN(sk_h); FD_PIN(sv_t); FD_PIN(sv_h); FD_PIN(sbt);
   FD_PIN(sm_scale); FD_PIN(batch); FD_PIN(G); FD_PIN(S); FD_PIN(P); FD_PIN(max_pages); FD_PIN(num_pages);
   FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(member_hb); FD_PIN(s_magic);
-  FD_PIN(s_shift);
+  FD_PIN(s_shift); FD_PIN(per_mask);
   // what the epilogue reads, so that it does not wait for the argument segment either
   FD_PIN(out); FD_PIN(lse); FD_PIN(so_b); FD_PIN(so_h); FD_PIN(so_s); FD_PIN(tickets); FD_PIN(mid_dtype);
   FD_PIN(vec_out); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
@@ -242,7 +244,8 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
   // per = ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)
-  const int per = (int)(((uint64_t)(uint32_t)(kv_len + a.S - 1) * a.s_magic) >> a.s_shift);
+  int per = (int)(((uint64_t)(uint32_t)(kv_len + a.S - 1) * a.s_magic) >> a.s_shift);
+  per = (per + a.per_mask) & ~a.per_mask;
   int64_t st = (int64_t)per * w.s;
   w.start = st > kv_len ? kv_len : (int)st;
   int64_t en = st + per;

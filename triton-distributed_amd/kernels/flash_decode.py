@@ -45,6 +45,8 @@ from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
 DEFAULT_KV_SPLITS = 32  # flash_decode.py:779
+SPLIT_ALIGN = 64        # tokens: the largest tile of the split kernels
+MAX_AUTO_KV_SPLITS = 128  # upper bound of the library's own choice (kv_split == -1, internal partials)
 
 
 def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size, split_kv=32, soft_cap=0.0):
@@ -90,7 +92,7 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 
 
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
-                 waves_per_block, seq_order_lens=None) -> FdParams:
+                 waves_per_block, seq_order_lens=None, split_align=0) -> FdParams:
     p = FdParams()
     p.q_heads = q.shape[1]
     p.kv_heads = k_cache.shape[2]
@@ -109,6 +111,7 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
     p.path = _PATHS[path]
     p.waves_per_block = waves_per_block
     p.seq_order_lens = seq_order_lens.data_ptr() if seq_order_lens is not None else None
+    p.split_align = split_align
     return p
 
 
@@ -129,6 +132,11 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     if (k_scale is None) != (v_scale is None):
         raise RuntimeError("k_scale and v_scale must be given together")
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
+    if kv_split == -1 and output_split is None:
+        # the caller left the split count to the library and cannot see the partials: long sequences may get more
+        # than the reference's 32 splits, as long as a split of a full-length sequence keeps 1024 tokens
+        capacity = block_table.shape[1] * page_size
+        num_splits = max(num_splits, min(MAX_AUTO_KV_SPLITS, capacity // 1024))
     lib = load_library()
     hstream = stream_handle(stream, q.device.index)
 
@@ -181,8 +189,9 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     if seq_order_lens is not None:
         assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
         assert seq_order_lens.numel() == batch
+    # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
-                     v_scale, path, waves_per_block, seq_order_lens)
+                     v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0)
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:
