@@ -92,7 +92,7 @@ typedef struct fd_params {
   const float* k_scale;     /* [Hkv] fp32 dequant scales, FD_FP8_E4M3 only         */
   const float* v_scale;     /* [Hkv]                                               */
   int32_t path;             /* fd_path                                             */
-  int32_t waves_per_block;  /* 0 = choose; else 1, 2, 4 or 8 wave64 per workgroup  */
+  int32_t waves_per_block;  /* 0 = choose; else 1, 2, 4 or 8 wave64 per (KV head, split) -- lowered where a kernel allows fewer */
   const int32_t* seq_order_lens; /* NULL, or [batch] with seq_order: kv_lens[seq_order[r]]
                                at index r (fd_kv_append writes it), so that a workgroup
                                fetches its sequence and its length in one round trip */

@@ -53,6 +53,13 @@ bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
   return dim_ok;
 }
 
+// Query-head slots of one head block of the MFMA kernels: 16 (one MFMA column block per wave), or 32 where the kernel
+// serves two column blocks per wave from one pass over K and V and the group is large enough to use them.
+int mfma_head_block(int head_dim, int group, int kv_dtype) {
+  const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
+  return (group > 16 && head_dim == 128 && kv16) ? 32 : 16;
+}
+
 // Launch-shape policy, from sweeps on one MI355X (256 CUs): the MFMA kernels stream best with about
 // 1024 waves in flight (16 KB of loads each), the VALU kernel with about 2048 (8 KB each), each walking
 // a long token range (every wave pays a fixed prologue / epilogue, and every split adds a partial for
@@ -64,26 +71,26 @@ constexpr int64_t kMaxTokensPerSplit = 4096;   // keeps a ragged batch balanceab
 
 // Waves per (KV head, split) when the caller does not choose: the smallest power of two that reaches
 // kTargetWaves, never more waves than tiles a split can have.
-int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, int64_t target) {
+int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, int64_t target, int max_waves) {
   int64_t tiles = (max_tokens_per_split + tile - 1) / tile;
   int w = 1;
-  while (w < 8 && head_splits * w < target && w * 2 <= tiles) w *= 2;
+  while (w < max_waves && head_splits * w < target && w * 2 <= tiles) w *= 2;
   const char* env = getenv("FD_WAVES_PER_BLOCK");
   if (env) {
     int e = atoi(env);
     if (e == 1 || e == 2 || e == 4 || e == 8) w = e;
   }
-  return w;
+  return w < max_waves ? w : max_waves;
 }
 
 // Adjacent KV heads per workgroup (one wave each): sibling waves fetch up to 512 contiguous bytes of
-// every token row together.  Bounded by 8 waves per workgroup and by keeping one workgroup per CU.
-int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_splits) {
+// every token row together.  Bounded by the waves a workgroup may have and by keeping one workgroup per CU.
+int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_splits, int max_waves) {
   int h = row_bytes > 0 ? 512 / row_bytes : 1;
   const char* env = getenv("FD_HEADS_PER_BLOCK");
   if (env && atoi(env) > 0) h = atoi(env);
   if (h < 1) h = 1;
-  while (h > 1 && (kv_heads % h != 0 || h * waves > 8 || head_splits / h < kMinWorkgroups)) h >>= 1;
+  while (h > 1 && (kv_heads % h != 0 || h * waves > max_waves || head_splits / h < kMinWorkgroups)) h >>= 1;
   return h;
 }
 
@@ -187,8 +194,9 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   int tile;
   if (use_mfma) {
-    a.hbsz = G < 16 ? G : 16;
-    a.nhb = (G + 15) / 16;
+    const int hb = mfma_head_block(D, G, p->kv_dtype);
+    a.hbsz = G < hb ? G : hb;
+    a.nhb = (G + hb - 1) / hb;
     tile = kv_fp8 ? (D == 256 ? 32 : 64) : (D == 64 ? 64 : (D == 256 ? 16 : 32));
   } else {
     a.hbsz = G >= 3 ? 4 : G;
@@ -198,15 +206,18 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
   const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
-  int waves = p->waves_per_block ? p->waves_per_block : choose_waves(wgs, max_tok_split, tile, use_mfma ? kTargetWaves : kTargetWavesValu);
+  // the two-block MFMA kernel needs the register file of a whole SIMD per wave: workgroups of at most 4 waves
+  const int max_waves = use_mfma && a.hbsz > 16 ? 4 : 8;
+  int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
+                                 : choose_waves(wgs, max_tok_split, tile, use_mfma ? kTargetWaves : kTargetWavesValu, max_waves);
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
   if (use_mfma && !fuse && a.nhb > 1) {
-    // more than 16 query heads per KV head: the head blocks of a KV head share a workgroup (largest divisor of
+    // more query heads per KV head than one wave serves: the head blocks of a KV head share a workgroup (largest divisor of
     // nhb that keeps the workgroup at 8 waves and the grid at one workgroup per CU), so that they read their
     // common K/V rows in step
-    int h = 8 / waves;
+    int h = max_waves / waves;
     const char* env = getenv("FD_HEADS_PER_BLOCK");   // same tuning override as for sibling KV heads
     if (env && atoi(env) > 0 && atoi(env) < h) h = atoi(env);
     while (h > 1 && (a.nhb % h != 0 || wgs / h < kMinWorkgroups)) --h;
@@ -215,7 +226,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
       a.member_hb = 1;
     }
   } else if (use_mfma && !fuse) {
-    a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs);
+    a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs, max_waves);
   }
   a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / a.hpw * a.nhb;
   a.nsub = waves;
@@ -223,7 +234,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS
   if (fuse) {  // the fused tail exchanges fp32 partials only
-    const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (use_mfma ? 16 : a.hbsz) * 4;
+    const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (use_mfma && a.hbsz < 16 ? 16 : a.hbsz) * 4;
     if (lse_lds <= kMaxLds / 2) {
       a.tickets = tail->tickets; a.fout = tail->out; a.flse = tail->lse_out;
       a.extra_out = tail->extra_out; a.extra_lse = tail->extra_lse;
@@ -323,7 +334,8 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
     return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0");
   const int G = p->q_heads / p->kv_heads;
   const bool mfma = mfma_shape_ok(p->head_dim, G, p->kv_dtype) && p->path != FD_PATH_VALU;
-  const int64_t nhb = mfma ? (G + 15) / 16 : (G + (G >= 3 ? 4 : G) - 1) / (G >= 3 ? 4 : G);
+  const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
+  const int64_t nhb = (G + hb - 1) / hb;
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
   // (1) enough splits to reach the target wave count with two (MFMA) or four (VALU) waves per head-split ...

@@ -41,11 +41,12 @@ struct SplitArgs {
   uint32_t div_magic, div_shift;  // n / P == (uint64(n) * div_magic) >> div_shift for 0 <= n < 2^31
   int32_t q_dtype, mid_dtype;
   int32_t nhb;      // head blocks per KV head
-  int32_t hbsz;     // query heads per head block
+  int32_t hbsz;     // query heads per head block (MFMA kernels: up to 16, or up to 32 with two column blocks per wave)
   int32_t hpw;      // adjacent KV heads per workgroup (one wave each; x token sub-ranges = waves)
   int32_t nsub;     // token sub-ranges of a split (waves per KV head); the workgroup has hpw * nsub waves
-  int32_t member_hb;  // 1: the hpw members of a workgroup are head blocks of ONE KV head (groups above 16 query
-                      // heads: the blocks read the same K/V rows in step, so the rows come from HBM once)
+  int32_t member_hb;  // 1: the hpw members of a workgroup are head blocks of ONE KV head (groups with more query
+                      // heads than a wave serves: the blocks read the same K/V rows in step, so the rows come
+                      // from HBM once)
   int32_t grid_x;   // workgroups per (sequence, split)
   int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)

@@ -4,9 +4,12 @@
 // (python/triton_dist/kernels/nvidia/flash_decode.py:130-239) for every GQA group
 // (the query heads of a KV head are padded to blocks of 16, the MFMA N).
 //
-// Decomposition: one workgroup per (sequence, split, KV head, block of <=16
+// Decomposition: one workgroup per (sequence, split, KV head, block of <=16*NB
 // query heads); its W waves take contiguous runs of 32-token tiles of the split
-// and are merged through LDS at the end.
+// and are merged through LDS at the end.  NB = 2 (groups above 16 query heads):
+// a wave serves two 16-head blocks from the same K and V registers -- the loads,
+// the LDS staging and the V transpose are shared, only the MFMAs and the softmax
+// are done per block.
 //
 // Per 32-token tile and wave (lane = 16*g + c):
 //   * 8 + 8 global_load_dwordx4: load i fetches, for every g, the full 256-byte
@@ -37,16 +40,19 @@ namespace {
 constexpr int kD = 128;
 constexpr int kTile = 32;         // tokens per tile
 constexpr int kKRow = 272;        // LDS pitch of a staged K row in bytes (256 + 16 pad)
-constexpr int kWaveLds = kTile * kKRow;  // 8704 B per wave, reused for the wave's partial result
-constexpr int kHB = 16;           // head slots per workgroup (MFMA N)
-static_assert(kWaveLds >= (kHB * kD + 2 * kHB) * 4, "partial result must fit in the K staging buffer");
+constexpr int kKTile = kTile * kKRow;   // 8704 B of staged K per wave
+// LDS per wave: the K staging buffer, reused for the wave's partial result (16*NB heads x (128 + 2) floats)
+constexpr int wave_lds(int nb) { return nb == 1 ? kKTile : (16 * nb * kD + 2 * 16 * nb) * 4; }
+static_assert(wave_lds(1) >= (16 * kD + 2 * 16) * 4 && wave_lds(2) >= kKTile, "partial result and K tile share the buffer");
 
 #ifndef FD_MFMA_OCC
 #define FD_MFMA_OCC
 #endif
 
-template <typename T, bool SOFTCAP>
-__global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const SplitArgs a) {
+template <typename T, bool SOFTCAP, int NB>
+__global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma16_kernel(const SplitArgs a) {
+  constexpr int kHB = 16 * NB;             // head slots per wave
+  constexpr int kWaveLds = wave_lds(NB);
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -61,18 +67,18 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
   const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 
-  const int head_in_group = w.hb * kHB + c;
-  const bool head_ok = head_in_group < a.G;
-  const int head = w.kvh * a.G + head_in_group;
-
-  // Q as the MFMA B operand: lane (g, c) holds Q[head c][32*ks + 8g .. +7].
-  u32x4 qop[4];
-  {
+  // Q as the MFMA B operand: lane (g, c) holds Q[head 16*nb + c][32*ks + 8g .. +7].
+  u32x4 qop[NB][4];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int head_in_group = w.hb * kHB + 16 * nb + c;
+    const bool head_ok = head_in_group < a.G;
+    const int head = w.kvh * a.G + head_in_group;
     const char* qp = (const char*)a.q + ((int64_t)w.b * a.sq_b + (int64_t)head * a.sq_h) * 2;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 z = {0u, 0u, 0u, 0u};
-      qop[ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
+      qop[nb][ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
     }
   }
 
@@ -115,11 +121,16 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
     for (int i = 0; i < 8; ++i) vraw[i] = load_stream_b128(vbase + (int64_t)rows[i] * v_pitch);
   };
 
-  float m = -INFINITY;  // running max of head c (identical in the 4 wave rows)
-  float l = 0.f;        // this lane's share of the running sum
-  f32x4 acc[8];         // acc[j][i] = O[head c][dim 32g + 8i + j]
+  float m[NB];          // running max of head 16*nb + c (identical in the 4 wave rows)
+  float l[NB];          // this lane's share of the running sum
+  f32x4 acc[NB][8];     // acc[nb][j][i] = O[head 16*nb + c][dim 32g + 8i + j]
 #pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    l[nb] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[nb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   int pg_next = 0, slot_next = 0;
 
@@ -146,72 +157,91 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- S^T = K . Q^T
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 s0[NB], s1[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) s0[nb] = s1[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 a0 = *(const u32x4*)(kb + c * kKRow + (4 * ks + g) * 16);
       u32x4 a1 = *(const u32x4*)(kb + (16 + c) * kKRow + (4 * ks + g) * 16);
-      s0 = Mma<T>::run(a0, qop[ks], s0);
-      s1 = Mma<T>::run(a1, qop[ks], s1);
-    }
-    // ---- online softmax (head c, tokens tau(g, 0..7))
-    float x[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x[i] = s0[i];
-      x[4 + i] = s1[i];
+      for (int nb = 0; nb < NB; ++nb) {
+        s0[nb] = Mma<T>::run(a0, qop[nb][ks], s0[nb]);
+        s1[nb] = Mma<T>::run(a1, qop[nb][ks], s1[nb]);
+      }
     }
+    // ---- online softmax (head 16*nb + c, tokens tau(g, 0..7))
     const int n0 = w.start + t * kTile;
     const bool full = n0 + kTile <= w.end;
+    u32x4 pop[NB];  // P^T as the B operand: element e <-> token tau(g, e)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float v = x[i];
-      if (SOFTCAP) {
-        v = fd_softcap(v * a.sm_scale, a.soft_cap, inv_cap) * FD_LOG2E;
-      } else {
-        v *= scale2;
+    for (int nb = 0; nb < NB; ++nb) {
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x[i] = s0[nb][i];
+        x[4 + i] = s1[nb][i];
       }
-      const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
-      x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
-    }
-    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m, mx);  // finite: every tile holds at least one valid token
-    const float alpha = fd_exp2(m - m_new);
-    float psum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      x[i] = fd_exp2(x[i] - m_new);
-      psum += x[i];
-    }
-    l = l * alpha + psum;
-    if (__any(m_new > m)) {
+      for (int i = 0; i < 8; ++i) {
+        float v = x[i];
+        if (SOFTCAP) {
+          v = fd_softcap(v * a.sm_scale, a.soft_cap, inv_cap) * FD_LOG2E;
+        } else {
+          v *= scale2;
+        }
+        const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
+        x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
+      }
+      float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m[nb], mx);  // finite: every tile holds at least one valid token
+      const float alpha = fd_exp2(m[nb] - m_new);
+      float psum = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] *= alpha;
-    }
-    m = m_new;
-    u32x4 pop;  // P^T as the B operand: element e <-> token tau(g, e)
+      for (int i = 0; i < 8; ++i) {
+        x[i] = fd_exp2(x[i] - m_new);
+        psum += x[i];
+      }
+      l[nb] = l[nb] * alpha + psum;
+      if (__any(m_new > m[nb])) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) pop[e] = Mma<T>::pack(x[2 * e], x[2 * e + 1]);
+        for (int j = 0; j < 8; ++j) acc[nb][j] *= alpha;
+      }
+      m[nb] = m_new;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pop[nb][e] = Mma<T>::pack(x[2 * e], x[2 * e + 1]);
+    }
 
-    // ---- V: transpose the lane's 8 tokens x 8 dims block into 8 A operands
-    u32x4 vop[8];
+    // ---- V: transpose the lane's 8 tokens x 8 dims block into 8 A operands, O^T += V^T . P^T.
+    // The next tile's V is requested as soon as the last raw V register has been consumed.  With two head
+    // blocks the operands are built in two halves to stay within the register file.
+    constexpr int kHalf = NB == 1 ? 8 : 4;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+    for (int j0 = 0; j0 < 8; j0 += kHalf) {
+      u32x4 vop[kHalf];
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        vop[j][e] = __builtin_amdgcn_perm(vraw[2 * e + 1][j >> 1], vraw[2 * e][j >> 1], sel);
+      for (int jj = 0; jj < kHalf; ++jj) {
+        const int j = j0 + jj;
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          vop[jj][e] = __builtin_amdgcn_perm(vraw[2 * e + 1][j >> 1], vraw[2 * e][j >> 1], sel);
+      }
+      if constexpr (HAS_NEXT) {
+        if (j0 + kHalf == 8) {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_v();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < kHalf; ++jj) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb][j0 + jj] = Mma<T>::run(vop[jj], pop[nb], acc[nb][j0 + jj]);
+      }
     }
-    if constexpr (HAS_NEXT) {
-      __builtin_amdgcn_sched_barrier(0);
-      issue_v();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // ---- O^T += V^T . P^T
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = Mma<T>::run(vop[j], pop, acc[j]);
   };
 
   if (t0 < t1) {
@@ -230,20 +260,25 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
   }
 
   // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
   wave_lds_fence();
   float* part = (float*)kb;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f32x4 lo = {acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
-    f32x4 hi = {acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
-    *(f32x4*)(part + c * kD + 32 * g + 8 * i) = lo;
-    *(f32x4*)(part + c * kD + 32 * g + 8 * i + 4) = hi;
-  }
-  if (g == 0) {
-    part[kHB * kD + c] = m;
-    part[kHB * kD + kHB + c] = l;
+  for (int nb = 0; nb < NB; ++nb) {
+    float lsum = l[nb];
+    lsum += __shfl_xor(lsum, 16);
+    lsum += __shfl_xor(lsum, 32);
+    const int h = 16 * nb + c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f32x4 lo = {acc[nb][0][i], acc[nb][1][i], acc[nb][2][i], acc[nb][3][i]};
+      f32x4 hi = {acc[nb][4][i], acc[nb][5][i], acc[nb][6][i], acc[nb][7][i]};
+      *(f32x4*)(part + h * kD + 32 * g + 8 * i) = lo;
+      *(f32x4*)(part + h * kD + 32 * g + 8 * i + 4) = hi;
+    }
+    if (g == 0) {
+      part[kHB * kD + h] = m[nb];
+      part[kHB * kD + kHB + h] = lsum;
+    }
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
@@ -253,19 +288,27 @@ __global__ void __launch_bounds__(512) FD_MFMA_OCC fd_split_mfma16_kernel(const 
 
 }  // namespace
 
+template <typename T>
+static auto pick_kernel(bool soft_cap, int nb) -> void (*)(const SplitArgs) {
+  if (nb == 2) return soft_cap ? fd_split_mfma16_kernel<T, true, 2> : fd_split_mfma16_kernel<T, false, 2>;
+  return soft_cap ? fd_split_mfma16_kernel<T, true, 1> : fd_split_mfma16_kernel<T, false, 1>;
+}
+
+// a.hbsz = query heads per head block: up to 16 (one MFMA column block per wave) or 32 (two)
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
   const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
   const unsigned block = 64u * waves;
-  size_t lds = (size_t)waves * kWaveLds;
+  const int nb = a.hbsz > 16 ? 2 : 1;
+  size_t lds = (size_t)waves * wave_lds(nb);
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
-    const size_t need = (size_t)(a.S + a.num_extra) * kHB * 4;
+    const size_t need = (size_t)(a.S + a.num_extra) * 16 * nb * 4;
     if (need > lds) lds = need;
   }
   void (*kern)(const SplitArgs) = nullptr;
   if (kv_dtype == FD_BF16) {
-    kern = soft_cap ? fd_split_mfma16_kernel<__bf16, true> : fd_split_mfma16_kernel<__bf16, false>;
+    kern = pick_kernel<__bf16>(soft_cap, nb);
   } else if (kv_dtype == FD_F16) {
-    kern = soft_cap ? fd_split_mfma16_kernel<_Float16, true> : fd_split_mfma16_kernel<_Float16, false>;
+    kern = pick_kernel<_Float16>(soft_cap, nb);
   } else {
     return FD_ERR_UNSUPPORTED;
   }
