@@ -42,6 +42,26 @@ def test_enums_and_params_struct_mirror_the_header(fd):
         assert pytype is expect, name
 
 
+def test_stand_alone_reference_binding_mirrors_the_same_structs(fd):
+    """reference_binding.py repeats the struct layouts on purpose (it imports nothing from the package): they must be
+    the package's, field for field, and its argtypes must be those of the package's binding."""
+    import importlib.util
+    path = os.path.join(ROOT, "triton-distributed_amd", "reference_binding.py")
+    spec = importlib.util.spec_from_file_location("fd_reference_binding_cpu", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    L = fd._lib
+    assert mod.FdParams._fields_ == L.FdParams._fields_ and ctypes.sizeof(mod.FdParams) == ctypes.sizeof(L.FdParams)
+    assert mod.FdQkPrep._fields_ == L.FdQkPrep._fields_ and ctypes.sizeof(mod.FdQkPrep) == ctypes.sizeof(L.FdQkPrep)
+    lib = fd.load_library()
+    for fn in ("fd_decode", "fd_kv_append"):
+        theirs, ours = getattr(mod._lib, fn).argtypes, getattr(lib, fn).argtypes
+        assert len(theirs) == len(ours), fn
+        for i, (a, b) in enumerate(zip(theirs, ours)):
+            both_pointers = hasattr(a, "contents") and hasattr(b, "contents")
+            assert a is b or both_pointers, (fn, i, a, b)
+
+
 def test_invalid_arguments_return_error_codes_without_touching_a_gpu(fd):
     lib = fd.load_library()
     L = fd._lib

@@ -69,17 +69,29 @@ constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = 4096;   // keeps a ragged batch balanceable by the dispatcher
 
+// Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
+// split) where the caller leaves the choice to the library) and FD_HEADS_PER_BLOCK (members per workgroup).
+int env_int(const char* name) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : 0;
+}
+int env_waves() {
+  static const int v = env_int("FD_WAVES_PER_BLOCK");
+  return v;
+}
+int env_heads() {
+  static const int v = env_int("FD_HEADS_PER_BLOCK");
+  return v;
+}
+
 // Waves per (KV head, split) when the caller does not choose: the smallest power of two that reaches
 // kTargetWaves, never more waves than tiles a split can have.
 int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, int64_t target, int max_waves) {
   int64_t tiles = (max_tokens_per_split + tile - 1) / tile;
   int w = 1;
   while (w < max_waves && head_splits * w < target && w * 2 <= tiles) w *= 2;
-  const char* env = getenv("FD_WAVES_PER_BLOCK");
-  if (env) {
-    int e = atoi(env);
-    if (e == 1 || e == 2 || e == 4 || e == 8) w = e;
-  }
+  const int e = env_waves();
+  if (e == 1 || e == 2 || e == 4 || e == 8) w = e;
   return w < max_waves ? w : max_waves;
 }
 
@@ -87,8 +99,7 @@ int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, in
 // every token row together.  Bounded by the waves a workgroup may have and by keeping one workgroup per CU.
 int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_splits, int max_waves) {
   int h = row_bytes > 0 ? 512 / row_bytes : 1;
-  const char* env = getenv("FD_HEADS_PER_BLOCK");
-  if (env && atoi(env) > 0) h = atoi(env);
+  if (env_heads() > 0) h = env_heads();
   if (h < 1) h = 1;
   while (h > 1 && (kv_heads % h != 0 || h * waves > max_waves || head_splits / h < kMinWorkgroups)) h >>= 1;
   return h;
@@ -218,8 +229,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     // nhb that keeps the workgroup at 8 waves and the grid at one workgroup per CU), so that they read their
     // common K/V rows in step
     int h = max_waves / waves;
-    const char* env = getenv("FD_HEADS_PER_BLOCK");   // same tuning override as for sibling KV heads
-    if (env && atoi(env) > 0 && atoi(env) < h) h = atoi(env);
+    if (env_heads() > 0 && env_heads() < h) h = env_heads();   // same tuning override as for sibling KV heads
     while (h > 1 && (a.nhb % h != 0 || wgs / h < kMinWorkgroups)) --h;
     if (h > 1) {
       a.hpw = h;
