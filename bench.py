@@ -273,7 +273,7 @@ def main():
     S_bound = S
     if S == -1:   # the library's own bound, as in the wrapper
         capacity = wl.block_table.shape[1] * wl.k_cache.shape[1]
-        S_bound = max(fk.DEFAULT_KV_SPLITS, min(fk.MAX_AUTO_KV_SPLITS, capacity // 1024))
+        S_bound = fk.auto_split_bound(capacity)
     p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_bound, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
                         wl.k_scale, wl.v_scale, args.path, args.waves)
     p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials

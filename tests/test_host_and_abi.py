@@ -197,17 +197,19 @@ def test_split_plan_policy(fd):
         p.num_pages, p.max_pages_per_seq, p.q_dtype, p.kv_dtype = 10, max_pages, L.FD_BF16, kv
         return lib.fd_plan_splits(ctypes.byref(p), B)
 
-    assert plan(8, 32, 8, 32, 512) == 8            # config 2: 1024 waves with 2 waves per (head, split)
+    assert plan(8, 32, 8, 32, 512) == 8            # config 2: 256 workgroups of 2 sibling heads x 2 waves
     assert plan(1, 32, 8, 32, 8192) == 32          # config 3: one sequence, all the splits the caller allows
     assert plan(64, 32, 8, 32, 2048) == 8          # config 4: <= 4096 tokens per split of a full-length sequence
     assert plan(32, 64, 8, 64, 1024, kv=L.FD_FP8_E4M3) == 4
-    assert plan(8, 32, 8, 32, 512, D=256) == 8     # head_dim 256 has an MFMA kernel too
+    assert plan(8, 32, 8, 32, 512, D=256) == 4     # head_dim 256: 512-byte rows, no sibling heads -> 256 workgroups
+    assert plan(8, 32, 8, 32, 512, D=64) == 16     # head_dim 64: four sibling heads per workgroup
     assert plan(8, 8, 8, 32, 512) == 8             # MHA runs on the MFMA kernels too
     assert plan(8, 8, 8, 32, 512, kv=L.FD_F32) == 8  # VALU path (fp32 cache): 2048 waves with 4 waves per (head, split)
     assert plan(2, 8, 8, 32, 512) == 32
-    assert plan(3, 32, 8, 32, 512) == 32           # 22 -> the next power of two
+    assert plan(3, 32, 8, 32, 512) == 32           # 21.3 -> the next power of two
     assert plan(3, 32, 8, 24, 512) == 16           # ... and down again when the caller allows fewer
-    assert plan(1, 96, 12, 128, 65536, P=1) == 64  # one long sequence, the library's own bound: 43 -> 64
+    assert plan(1, 96, 12, 128, 65536, P=1) == 128  # 12 KV heads: 64 splits would be 1.5 workgroups per CU, 128 are 3
+    assert plan(1, 8, 1, 256, 65536) == 256        # one KV head: one split per CU
     assert plan(1, 96, 12, 128, 1 << 20, P=1) == 128
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1

@@ -348,18 +348,38 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   const int64_t nhb = (G + hb - 1) / hb;
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
-  // (1) enough splits to reach the target wave count with two (MFMA) or four (VALU) waves per head-split ...
-  const int64_t per_split = mfma ? 2 * groups : 4 * groups;
-  const int64_t target = mfma ? kTargetWaves : kTargetWavesValu;
-  int64_t s_fill = (target + per_split - 1) / per_split;
-  // (2) ... and enough that no split of a full-length sequence is longer than kMaxTokensPerSplit
-  int64_t s_bal = (max_tokens + kMaxTokensPerSplit - 1) / kMaxTokensPerSplit;
-  int64_t s = s_fill > s_bal ? s_fill : s_bal;
-  // (3) a power of two: with sequence lengths that are powers of two (or multiples of large ones) every split then
-  // starts on a tile boundary and the waves of a workgroup get equal runs
-  int64_t pow2 = 1;
-  while (pow2 < s) pow2 <<= 1;
-  s = pow2;
+  int64_t s;
+  if (mfma) {
+    // (1) one workgroup per CU at the full member width (sibling KV heads, or head blocks of one KV head): measured
+    // over head dims, cache dtypes and batch sizes, 256 workgroups x 4 waves beats 512 x 2 and 128 x 8 ...
+    int members = 1;
+    if (nhb > 1) {
+      for (int h = 4; h > 1; --h)
+        if (nhb % h == 0) { members = h; break; }
+    } else {
+      const int row_bytes = p->head_dim * dtype_size(p->kv_dtype);
+      members = row_bytes > 0 && row_bytes < 512 ? 512 / row_bytes : 1;
+      while (members > 1 && p->kv_heads % members != 0) members >>= 1;
+    }
+    s = 1;
+    while (s * groups < kMinWorkgroups * members) s <<= 1;
+    // (2) ... and, for a single sequence (equal work items, one round), a whole number of workgroups per CU or at
+    // least four: 1.5 workgroups per CU take as long as 2
+    while (batch == 1 && s < p->num_splits && (s * groups / members) % kMinWorkgroups != 0 &&
+           s * groups / members < 4 * kMinWorkgroups)
+      s <<= 1;
+  } else {
+    // the VALU kernel keeps half as many bytes in flight per wave: twice the waves, four per (KV head, split)
+    s = 1;
+    while (s * 4 * groups < kTargetWavesValu) s <<= 1;
+  }
+  // (3) in a batch, enough splits that no split of a full-length sequence is longer than kMaxTokensPerSplit: the
+  // dispatcher evens out ragged lengths with them
+  if (batch > 1) {
+    while (s * kMaxTokensPerSplit < max_tokens) s <<= 1;
+  }
+  // Powers of two throughout: with sequence lengths that are powers of two (or multiples of large ones) every split
+  // then starts on a tile boundary and the waves of a workgroup get equal runs.
   while (s > p->num_splits) s >>= 1;
   if (s < 1) s = 1;
   return (int)s;

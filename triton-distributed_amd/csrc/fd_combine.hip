@@ -3,14 +3,18 @@
 // fd_combine_kernel replaces the reference's three combine kernels
 // (python/triton_dist/kernels/nvidia/flash_decode.py:308-360 plain, :393-449
 // intra-rank with merged LSE, :482-532 inter-rank).  The reference walks the
-// partials sequentially with a running max.  Here one 256-thread workgroup per
-// (sequence, head) first brings all partial LSEs into LDS (one load per
-// thread), every thread derives M = max and the weights w_s = e^{LSE_s - M}
-// from there, and then the threads -- laid out as ROWS row groups x D/4
-// column groups -- accumulate sum_s w_s * O_s with 128-bit loads that do not
-// depend on each other.  The row groups are summed through LDS.  The value is
-// the reference's: out = sum_s softmax(LSE)_s * O_s, LSE = logsumexp_s(LSE_s);
-// the cost is two dependent memory round trips instead of S.
+// partials sequentially with a running max.  Here a 256-thread workgroup per
+// (sequence, head, column chunk) first brings all partial LSEs into LDS (one
+// load per thread), every thread derives M = max and the weights
+// w_s = e^{LSE_s - M} from there, and then the threads -- laid out as ROWS row
+// groups x CG column groups of 4 columns -- accumulate sum_s w_s * O_s with
+// 128-bit loads that do not depend on each other.  The row groups are summed
+// through LDS.  The value is the reference's: out = sum_s softmax(LSE)_s * O_s,
+// LSE = logsumexp_s(LSE_s); the cost is two dependent memory round trips
+// instead of S.  CG is chosen per launch: D/4 (one workgroup per row of the
+// output) down to 4 (D/16 workgroups per row, 64 row groups), so that a step
+// with few output rows and many partials (one long sequence, few heads)
+// still spreads over the chip and needs few loads per thread.
 #include "fd_common.h"
 
 namespace {
@@ -19,17 +23,29 @@ constexpr int kCombineThreads = 256;
 constexpr int kMaxPartials = 1024;  // LSEs staged in LDS per pass
 constexpr int kPrefetch = 8;        // partial rows a thread requests before the weights are known
 
+// max of v[0..n) (LDS), the same value in every lane: a strided scan per lane, then a butterfly over the wave
+__device__ __forceinline__ float wave_max_of(const float* v, int n) {
+  float m = -INFINITY;
+  for (int i = threadIdx.x & 63; i < n; i += 64) m = fmaxf(m, v[i]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  return m;
+}
+
 template <int D>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const CombineArgs a) {
-  constexpr int CG = D / 4;                    // column groups (one 128-bit chunk of fp32 each)
-  constexpr int ROWS = kCombineThreads / CG;   // partial rows in flight per pass
+  const int CG = 1 << a.cg_shift;              // column groups of this workgroup (one 128-bit chunk of fp32 each)
+  const int ROWS = kCombineThreads >> a.cg_shift;   // partial rows in flight per pass
+  const int chunks = (D / 4) >> a.cg_shift;    // workgroups per output row (a power of two)
   __shared__ float s_lse[kMaxPartials];
-  __shared__ __align__(16) float s_acc[ROWS][D];
-  __shared__ float s_l[ROWS];
+  __shared__ __align__(16) float s_acc[kCombineThreads * 4];   // [ROWS][4 * CG]
+  __shared__ float s_l[kCombineThreads / 4];                   // [ROWS], ROWS <= 64
 
   const int tid = threadIdx.x;
-  const int b = blockIdx.x / a.Hq;
-  const int h = blockIdx.x - b * a.Hq;
+  const int row = blockIdx.x / chunks;
+  const int col0 = (blockIdx.x - row * chunks) * 4 * CG;   // first column of this workgroup
+  const int b = row / a.Hq;
+  const int h = row - b * a.Hq;
   const int S = a.num_partials;
   const int NP = S + a.num_extra;
   const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
@@ -55,8 +71,8 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
     return load_as_f32(a.mid_o, mid_base + (int64_t)s * a.s_ms + D, a.mid_dtype);
   };
 
-  const int r = tid / CG;
-  const int c = tid - r * CG;
+  const int r = tid >> a.cg_shift;
+  const int c = col0 / 4 + (tid - (r << a.cg_shift));   // 128-bit column group within the row
   const bool vec_mid = a.mid_dtype == FD_F32 && a.vec_mid;
   auto load_row = [&](int s) -> f32x4 {   // this thread's 4 columns of partial s
     f32x4 o;
@@ -89,7 +105,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
     }
     for (int i = tid; i < NP; i += kCombineThreads) s_lse[i] = partial_lse(i);
     __syncthreads();
-    for (int i = 0; i < NP; ++i) M = fmaxf(M, s_lse[i]);
+    M = wave_max_of(s_lse, NP);
     if (M > -INFINITY) {
 #pragma unroll
       for (int p = 0; p < kPrefetch; ++p) {
@@ -105,8 +121,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
       __syncthreads();
       for (int i = tid; i < cnt; i += kCombineThreads) s_lse[i] = partial_lse(p0 + i);
       __syncthreads();
-      float m_pass = -INFINITY;
-      for (int i = 0; i < cnt; ++i) m_pass = fmaxf(m_pass, s_lse[i]);
+      const float m_pass = wave_max_of(s_lse, cnt);
       const float m_new = fmaxf(M, m_pass);
       if (m_new == -INFINITY) continue;  // nothing valid so far (uniform)
       const float resc = __expf(M - m_new);  // 0 on the first valid pass
@@ -121,20 +136,19 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
       }
     }
   }
-  *(f32x4*)&s_acc[r][4 * c] = acc;
-  if (c == 0) s_l[r] = L;
+  *(f32x4*)&s_acc[tid * 4] = acc;   // row r, columns 4 * (tid % CG) .. + 3 of the chunk
+  if ((tid & (CG - 1)) == 0) s_l[r] = L;
   __syncthreads();
-  if (tid < D) {
+  if (tid < 4 * CG) {
     float o = 0.f, Lsum = 0.f;
-#pragma unroll
     for (int i = 0; i < ROWS; ++i) {
-      o += s_acc[i][tid];
+      o += s_acc[i * 4 * CG + tid];
       Lsum += s_l[i];
     }
     const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
     const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
-    store_from_f32(a.out, out_base + tid, a.out_dtype, o * inv);
-    if (tid == 0) {
+    store_from_f32(a.out, out_base + col0 + tid, a.out_dtype, o * inv);
+    if (tid == 0 && col0 == 0) {
       const float lse = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
       if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, lse);
       if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = lse;
@@ -223,11 +237,22 @@ __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restr
 
 }  // namespace
 
-int fd_launch_combine(hipStream_t stream, const CombineArgs& a) {
-  const unsigned grid = (unsigned)a.batch * a.Hq;
+int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
+  CombineArgs a = args;
+  const int64_t rows = (int64_t)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
   const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 &&
                      a.num_partials <= kSmallMax && a.mid_dtype == FD_F32 && a.vec_mid;
+  // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
+  // one workgroup per CU and a thread would still have more than two partials to walk.
+  int cg = a.D / 4;
+  const int64_t np = (int64_t)a.num_partials + a.num_extra;
+  while (!small && cg > 4 && rows * (a.D / 4 / cg) < 256 && np > 2 * (kCombineThreads / cg)) cg >>= 1;
+  a.cg_shift = 0;
+  while ((1 << a.cg_shift) < cg) ++a.cg_shift;
+  const int64_t wgs = small ? rows : rows * (a.D / 4 / cg);
+  if (wgs >= ((int64_t)1 << 31)) return FD_ERR_TOO_LARGE;
+  const unsigned grid = (unsigned)wgs;
   switch (a.D) {
     case 64: kern = small ? fd_combine_small_kernel<64> : fd_combine_kernel<64>; break;
     case 128: kern = small ? fd_combine_small_kernel<128> : fd_combine_kernel<128>; break;

@@ -74,6 +74,7 @@ struct CombineArgs {
   int64_t s_mb, s_mh, s_ms, s_ob, s_oh;
   int32_t batch, Hq, D, num_partials, num_extra, mode, mid_dtype, out_dtype;
   int32_t vec_mid;  // 1: every mid_o row start is 16-byte aligned (128-bit loads allowed)
+  int32_t cg_shift; // log2 of the 128-bit column groups a workgroup of the general kernel covers (set by the launcher)
   int32_t per_mask;           // as SplitArgs::per_mask, for the validity of split ranges
   int32_t all_slots_written;  // 1: the partials come from this library's split kernel in the same call, which
                               // writes every slot (empty splits as out = 0, lse = -inf)

@@ -46,7 +46,7 @@ from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
 DEFAULT_KV_SPLITS = 32  # flash_decode.py:779
 SPLIT_ALIGN = 64        # tokens: the largest tile of the split kernels
-MAX_AUTO_KV_SPLITS = 128  # upper bound of the library's own choice (kv_split == -1, internal partials)
+MAX_AUTO_KV_SPLITS = 256  # upper bound of the library's own choice (kv_split == -1, internal partials)
 
 
 def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size, split_kv=32, soft_cap=0.0):
@@ -71,6 +71,12 @@ def get_combine_kv_algo_info(split_kv=32, v_head_dim=128, block_dv=512):
 
 
 get_triton_combine_kv_algo_info = get_combine_kv_algo_info
+
+
+def auto_split_bound(capacity: int) -> int:
+    """Upper bound of the split count when the caller leaves it to the library (``kv_split == -1`` and no
+    ``output_split``): the reference's 32 (flash_decode.py:779), more for block tables of more than 16384 tokens."""
+    return max(DEFAULT_KV_SPLITS, min(MAX_AUTO_KV_SPLITS, capacity // 512))
 
 
 def _require_cuda(*tensors):
@@ -134,9 +140,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
     if kv_split == -1 and output_split is None:
         # the caller left the split count to the library and cannot see the partials: long sequences may get more
-        # than the reference's 32 splits, as long as a split of a full-length sequence keeps 1024 tokens
-        capacity = block_table.shape[1] * page_size
-        num_splits = max(num_splits, min(MAX_AUTO_KV_SPLITS, capacity // 1024))
+        # than the reference's 32 splits, as long as a split of a full-length sequence keeps 512 tokens
+        num_splits = auto_split_bound(block_table.shape[1] * page_size)
     lib = load_library()
     hstream = stream_handle(stream, q.device.index)
 
