@@ -33,6 +33,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (2 = Llama-3-8B shape, the one the metric is quoted on)")
     ap.add_argument("--pools", type=int, default=4, help="independent KV pools the steps rotate over")
+    ap.add_argument("--clock-ramp-ms", type=float, default=250.0,
+                    help="untimed run of the step before the warm-up steps, so that an idle GPU reaches its clocks")
     ap.add_argument("--variant", default="plain", choices=["plain", "persistent"])
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
@@ -251,6 +253,16 @@ def main():
         return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
 
     # ---- whole-step timing
+    # An idle GPU takes a while to reach its clocks, longer than a warm-up of a few milliseconds: run the step untimed
+    # for a quarter of a second first (the first measurement on a freshly acquired machine otherwise reads ~4 % low
+    # against the same command a minute later).
+    t_ramp = time.perf_counter()
+    i_ramp = 0
+    while time.perf_counter() - t_ramp < args.clock_ramp_ms * 1e-3:
+        for _ in range(50):
+            step(i_ramp)
+            i_ramp += 1
+        torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -354,6 +366,7 @@ def main():
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        "clock_ramp_ms": args.clock_ramp_ms,
         "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "kernel_us": round(split_us, 3)},

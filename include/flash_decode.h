@@ -214,11 +214,13 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  * not look at.  NUM_KV_SPLITS is a tuning constant in the reference (flash_decode.py:779:
  * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
  * the partial workspace is internal, fewer and longer splits mean fewer workgroup
- * prologues and fewer partials for the combine.  Returns min(params->num_splits, the split
- * count that (1) reaches about 1024 waves with two waves per (KV head, split) on the MFMA
- * kernels, or about 2048 with four on the VALU kernel, and (2) keeps every split of a
- * full-length sequence at or below 4096 tokens, rounded up to a power of two and then
- * down to at most params->num_splits), or a negative fd_status.
+ * prologues and fewer partials for the combine.  Returns a power of two, at most
+ * params->num_splits: the smallest split count that (1) gives one workgroup per CU (256) with
+ * the workgroup at its full width (sibling KV heads that share 512 bytes of a token row, or head
+ * blocks of one KV head), raised (2) until the workgroups are a whole number per CU or at
+ * least four per CU, as long as a split of a full-length sequence keeps 512 tokens, and (3) in
+ * a batch until no split of a full-length sequence exceeds 4096 tokens (VALU kernel: about
+ * 2048 waves with four per split instead of (1) and (2)); or a negative fd_status.
  * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
  * params->num_splits splits with the reference's ranges.
  */

@@ -363,10 +363,10 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
     }
     s = 1;
     while (s * groups < kMinWorkgroups * members) s <<= 1;
-    // (2) ... and, for a single sequence (equal work items, one round), a whole number of workgroups per CU or at
-    // least four: 1.5 workgroups per CU take as long as 2
-    while (batch == 1 && s < p->num_splits && (s * groups / members) % kMinWorkgroups != 0 &&
-           s * groups / members < 4 * kMinWorkgroups)
+    // (2) ... and a whole number of workgroups per CU, or at least four, while a split of a full-length sequence
+    // keeps 512 tokens: equal work items run in one round, and 1.5 workgroups per CU take as long as 2
+    while (s < p->num_splits && (s * groups / members) % kMinWorkgroups != 0 &&
+           s * groups / members < 4 * kMinWorkgroups && 2 * s * 512 <= max_tokens)
       s <<= 1;
   } else {
     // the VALU kernel keeps half as many bytes in flight per wave: twice the waves, four per (KV head, split)

@@ -52,7 +52,9 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         self.page_size = page_size
         self.soft_cap = soft_cap
         self.scale = scale
-        self.kv_split = 32
+        # The reference fixes 32 splits (sp_flash_decode_layer.py:62).  The partials never leave this layer, so the
+        # count is left to the library: 32 for short shards, up to 256 for long ones.
+        self.kv_split = -1
         self.max_allowed_batch = max_allowed_batch
         self.stages = stages
         self.partial_dtype = partial_dtype
