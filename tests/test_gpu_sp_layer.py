@@ -146,6 +146,36 @@ def test_many_partials_and_extras(fd):
     assert_lse_close(lse_out, torch.logsumexp(lses.double(), 0).float(), rtol=1e-5)
 
 
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("rows,R", [((1, 1), 17), ((1, 8), 40), ((1, 8), 256), ((2, 3), 200), ((1, 2), 1100),
+                                    ((1, 96), 128), ((4, 64), 33)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_combine_over_every_workgroup_width(fd, D, rows, R, dtype):
+    """Few output rows and many partials make the combine kernel split a row over several workgroups (down to 16
+    columns each); every width must give the closed form sum_r softmax(lse)_r * out_r, with invalid ranks skipped."""
+    B, Hq = rows
+    g = torch.Generator().manual_seed(100 * R + D + B)
+    outs = torch.randn(R, B, Hq, D, generator=g)
+    lses = torch.randn(R, B, Hq, generator=g) * 3 + 7
+    packed = torch.cat([outs, lses[..., None]], -1).to(dtype)
+    lens = torch.ones(R, B, dtype=torch.int32)
+    lens[torch.rand(R, B, generator=g) < 0.2] = 0
+    lens[0] = 1
+    poisoned = packed.clone()
+    poisoned[lens == 0] = float("nan")
+    final = torch.empty(B, Hq, D, dtype=dtype, device=DEV)
+    lse_out = torch.empty(B, Hq, dtype=torch.float32, device=DEV)
+    fd.inter_rank_combine(poisoned.to(DEV), final, lens.to(DEV), lse_out=lse_out)
+    torch.cuda.synchronize()
+    o64, l64 = packed[..., :D].double(), packed[..., D].double()
+    l64 = l64.masked_fill((lens == 0)[:, :, None], float("-inf"))
+    wts = torch.softmax(l64, 0)
+    ref = (wts[..., None] * o64.masked_fill((lens == 0)[:, :, None, None], 0.0)).sum(0).float()
+    f32 = dtype == torch.float32
+    assert_out_close(final, ref, atol=1e-5 if f32 else 2e-2)
+    assert_lse_close(lse_out, torch.logsumexp(l64, 0).float(), rtol=1e-5 if f32 else 1e-3)
+
+
 def test_raw_c_abi_split_then_combine(fd):
     """fd_split_kv and fd_combine called directly through ctypes with the reference's packed layouts."""
     lib = fd.load_library()
