@@ -243,13 +243,9 @@ def main():
     if args.exact_splits:
         kw["plan_splits"] = False
     fn = fd.gqa_fwd_batch_decode_persistent if args.variant == "persistent" else fd.gqa_fwd_batch_decode
-    if args.variant == "persistent":
-        kw["seq_order"] = torch.empty(B, dtype=torch.int32, device=dev)
 
-    def step(i):
+    def step(i):   # persistent: the scheduling launch is part of the step (inside the wrapper)
         k, v = pools[i % len(pools)]
-        if args.variant == "persistent":   # the scheduler is part of the step
-            fd.schedule_sequences(wl.kv_lens, out=kw["seq_order"])
         return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
 
     # ---- whole-step timing
@@ -290,6 +286,8 @@ def main():
                         wl.k_scale, wl.v_scale, args.path, args.waves)
     p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials
     S_eff = S_bound if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
+    if not args.exact_splits:
+        p.split_adapt = lib.fd_plan_min_splits(byref(p), B)
     p.num_splits = S_eff
     n_o = B * Hq * S_eff * D
     split_ws = workspace if workspace is not None else torch.empty(B * Hq * S_eff * (D + 1), dtype=torch.float32,
@@ -297,7 +295,15 @@ def main():
     mid = split_ws[:n_o].view(B, Hq, S_eff, D)
     lse_split = split_ws[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
     hstream = torch.cuda.current_stream().cuda_stream
-    order_ptr = kw["seq_order"].data_ptr() if args.variant == "persistent" else None
+    order_ptr = None
+    if args.variant == "persistent" and not args.exact_splits and S_eff > 1 and p.split_adapt > 0 and B <= fk.MAX_ITEM_BATCH:
+        # the issue order the scheduled step uses: (sequence, range) items, computed once for this leg
+        items = fk.item_order_buffer(B, S_eff, dev)
+        fd._lib.check(lib.fd_schedule_items(hstream, wl.kv_lens.data_ptr(), B, items.data_ptr(), byref(p)))
+        p.seq_order_items = 1
+        order_ptr = items.data_ptr()
+    elif args.variant == "persistent":
+        order_ptr = fd.schedule_sequences(wl.kv_lens).data_ptr()
 
     def split_only(i):
         k, v = pools[i % len(pools)]

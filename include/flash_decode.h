@@ -101,6 +101,18 @@ typedef struct fd_params {
                                so that splits start on tile boundaries (trailing splits may be
                                empty).  The result of a step is the same; the partials are not
                                the reference's.  fd_combine applies the same rule.          */
+  int32_t split_adapt;      /* 0: every sequence is cut into num_splits ranges (the reference).
+                               k > 0 (a power of two; needs split_align > 0): a range of a sequence
+                               of n tokens holds max(ceil(n / num_splits), min(ceil(n / k), 1024))
+                               tokens -- k ranges up to k * 1024 tokens, 1024-token ranges up to
+                               num_splits * 1024, num_splits ranges beyond -- so a block table
+                               sized for the longest context does not cut a short sequence into
+                               slivers.  The other ranges of the sequence are empty; with more
+                               than 16 splits fd_decode does not even write their partials.
+                               fd_plan_min_splits gives k.  fd_combine applies the same rule. */
+  int32_t seq_order_items;  /* 0: seq_order / seq_order_out is a per-sequence order ([batch], see
+                               fd_schedule and fd_kv_append).  1: it is the work-item order of
+                               fd_schedule_items, int32 [2 * batch * num_splits].             */
 } fd_params;
 
 /*
@@ -210,6 +222,20 @@ FD_API int fd_decode(void* stream, const void* q, const void* k_cache, const voi
 FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* seq_order);
 
 /*
+ * Kernel (3), per work item: the issue order of the (sequence, range) items of a decode step with
+ * params->num_splits, split_align and split_adapt, for batches of up to 1024 sequences.
+ * item_order[k], k < batch * num_splits, = sequence | range << 16: first the non-empty ranges, sequence by
+ * sequence in descending (tokens per range, length) order (largest item first), then the empty ranges;
+ * item_order[batch * num_splits + k] = the length of item k's sequence.  fd_decode / fd_split_kv take it as
+ * seq_order with params->seq_order_items = 1 (same num_splits, split_align, split_adapt, max_pages_per_seq and
+ * page_size; kv_lens unchanged in between).  With ranges that follow each sequence's own length this is what keeps the
+ * busy workgroups of a ragged batch contiguous in issue order AND largest-first.  The reference has no counterpart
+ * (static round-robin, flash_decode.py:632-640).
+ */
+FD_API int fd_schedule_items(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* item_order,
+                             const fd_params* params);
+
+/*
  * How many splits the library would use for a decode step whose partials the caller does
  * not look at.  NUM_KV_SPLITS is a tuning constant in the reference (flash_decode.py:779:
  * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
@@ -225,6 +251,15 @@ FD_API int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int3
  * params->num_splits splits with the reference's ranges.
  */
 FD_API int fd_plan_splits(const fd_params* params, int32_t batch);
+
+/*
+ * The part of fd_plan_splits' count that the shape needs to fill the chip (its rules 1 and 2, or the VALU
+ * rule), without the part that only bounds the length of a split in a batch: the value for
+ * fd_params.split_adapt.  No counterpart in the reference (one split count for all sequences,
+ * flash_decode.py:193-195).  Returns the count (a power of two >= 1, not clamped to params->num_splits) or a negative
+ * fd_status.
+ */
+FD_API int fd_plan_min_splits(const fd_params* params, int32_t batch);
 
 /*
  * What the reference's attention block does to q and k between the QKV projection and the

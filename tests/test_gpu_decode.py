@@ -467,7 +467,7 @@ def test_errors_are_reported_not_fatal(fd):
 
 
 # ---- HIP graph capture: the whole step (scheduler + split + combine) replays from a graph
-@pytest.mark.parametrize("variant", ["plain", "persistent"])
+@pytest.mark.parametrize("variant", ["plain", "persistent", "persistent_items"])
 def test_graph_capture_and_replay(fd, variant):
     wl = _grid_workload(fd, [1320, 463, 2049, 77], (32, 8), 128, 16, torch.bfloat16, 0, seed=81).to(DEV)
     B = 4
@@ -475,10 +475,10 @@ def test_graph_capture_and_replay(fd, variant):
     lse = torch.empty(B, 32, dtype=torch.float32, device=DEV)
     ws = torch.empty(B * 32 * 32 * 129, dtype=torch.float32, device=DEV)
     order = torch.empty(B, dtype=torch.int32, device=DEV)
-    fn = fd.gqa_fwd_batch_decode_persistent if variant == "persistent" else fd.gqa_fwd_batch_decode
+    fn = fd.gqa_fwd_batch_decode if variant == "plain" else fd.gqa_fwd_batch_decode_persistent
 
     def step():
-        kw = {}
+        kw = {}   # persistent_items: the wrapper schedules (sequence, range) items itself
         if variant == "persistent":
             fd.schedule_sequences(wl.kv_lens, out=order)
             kw["seq_order"] = order
@@ -510,6 +510,88 @@ def test_graph_capture_and_replay(fd, variant):
     ref, ref_lse = oracle_decode(wl.to("cpu"))
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
+
+
+# ---- block tables sized for the longest context: the split count follows each sequence's own length
+@pytest.mark.parametrize("capacity", [8192, 131072, 1048576])
+@pytest.mark.parametrize("kind", ["bf16", "fp16_d256", "fp8", "fp32_valu", "bf16_d64", "g32"])
+@pytest.mark.parametrize("batch", [5, 70])
+def test_short_sequences_in_a_block_table_sized_for_long_contexts(fd, capacity, kind, batch):
+    import random
+    rng = random.Random(capacity + batch)
+    lens = [rng.choice([0, 1, 37, 64, 1000, 4096, 4097, 5000, 8192]) for _ in range(batch)]
+    lens[0], lens[1] = 5000, 0
+    Hq, Hkv, D, dtype, fp8 = {"bf16": (32, 8, 128, torch.bfloat16, False), "fp16_d256": (16, 4, 256, torch.float16, False),
+                              "fp8": (64, 8, 128, torch.bfloat16, True), "fp32_valu": (8, 4, 128, torch.float32, False),
+                              "bf16_d64": (32, 8, 64, torch.bfloat16, False), "g32": (32, 1, 128, torch.bfloat16, False)}[kind]
+    P = 16
+    wl = fd.utils.make_paged_workload("wide_table", lens, Hq, Hkv, D, P, dtype, -1, seed=29, fp8_kv=fp8)
+    # widen the table: entries beyond a sequence's pages are garbage, as in a serving engine's preallocated table
+    gen = torch.Generator().manual_seed(3)
+    wide = torch.randint(-5, 1 << 30, (batch, capacity // P), generator=gen, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        used = -(-n // P)
+        wide[b, :used] = wl.block_table[b, :used]
+    wl.block_table = wide
+    ref, ref_lse = oracle_decode(wl)
+    f32 = dtype == torch.float32
+    for kv_split in (-1, 32, 8):
+        wl.kv_split = kv_split
+        out, lse = run_decode(fd, wl)
+        assert_out_close(out, ref, atol=2e-4 if f32 else 2e-2)
+        assert_lse_close(lse, ref_lse, rtol=1e-5 if f32 else 1e-3)
+    # the merged LSE column and extra partials go through the same ranges
+    res, _ = run_decode(fd, wl, variant="intra")
+    assert_out_close(res[..., :D], ref, atol=2e-4 if f32 else 2e-2)
+    assert_lse_close(res[..., D].float(), ref_lse, rtol=1e-5 if f32 else 1e-2)
+
+
+# ---- scheduled issue order by (sequence, range) items: the scheduling launch, the append-fused one, the raw ABI
+@pytest.mark.parametrize("capacity", [4096, 65536])
+@pytest.mark.parametrize("kind", ["bf16", "fp8", "fp32_valu"])
+@pytest.mark.parametrize("batch", [3, 40, 300])
+def test_item_schedule_matches_oracle_and_is_a_permutation(fd, capacity, kind, batch):
+    import random
+    from ctypes import byref
+    rng = random.Random(7 * capacity + batch)
+    lens = [rng.choice([0, 1, 63, 64, 65, 700, 1024, 1025, 2500, 4096]) for _ in range(batch)]
+    lens[0] = 4096
+    Hq, Hkv, D, dtype, fp8 = {"bf16": (32, 8, 128, torch.bfloat16, False), "fp8": (64, 8, 128, torch.bfloat16, True),
+                              "fp32_valu": (8, 4, 128, torch.float32, False)}[kind]
+    P = 16
+    wl = fd.utils.make_paged_workload("items", lens, Hq, Hkv, D, P, dtype, -1, seed=31, fp8_kv=fp8)
+    wide = torch.zeros((batch, capacity // P), dtype=torch.int32)
+    wide[:, :wl.block_table.shape[1]] = wl.block_table
+    wl.block_table = wide
+    ref, ref_lse = oracle_decode(wl)
+    f32 = dtype == torch.float32
+    out, lse = run_decode(fd, wl, variant="persistent")
+    assert_out_close(out, ref, atol=2e-4 if f32 else 2e-2)
+    assert_lse_close(lse, ref_lse, rtol=1e-5 if f32 else 1e-3)
+    # the raw scheduler: a permutation of all (sequence, range) pairs, non-empty ranges first and largest first
+    fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
+    g = wl.to(DEV)
+    S, adapt = fk.plan_decode(g.q, g.k_cache, g.block_table, -1, k_scale=g.k_scale, v_scale=g.v_scale)
+    if S == 1 or adapt == 0:
+        return
+    p = fk._make_params(g.q, g.k_cache, g.block_table, S, 0.0, 0, 0, g.k_scale, g.v_scale, "auto", 0, None,
+                        fk.SPLIT_ALIGN, adapt)
+    items = fk.item_order_buffer(batch, S, DEV)
+    fd._lib.check(fd.load_library().fd_schedule_items(None, g.kv_lens.data_ptr(), batch, items.data_ptr(), byref(p)))
+    torch.cuda.synchronize()
+    it = items.cpu().view(2, batch * S)
+    seq, rng_ = (it[0] & 0xFFFF).tolist(), ((it[0] >> 16) & 0xFFFF).tolist()
+    assert sorted(zip(seq, rng_)) == [(b, s) for b in range(batch) for s in range(S)]
+    assert it[1].tolist() == [lens[b] for b in seq]
+
+    def per(n):   # the library's range rule (include/flash_decode.h, fd_params.split_adapt)
+        v = max(-(-n // S), min(-(-n // adapt), 1024))
+        return -(-v // fk.SPLIT_ALIGN) * fk.SPLIT_ALIGN
+    busy = [per(lens[b]) * s < lens[b] for b, s in zip(seq, rng_)]
+    n_busy = sum(busy)
+    assert all(busy[:n_busy]) and not any(busy[n_busy:])
+    sizes = [per(lens[b]) for b in seq[:n_busy]]
+    assert sizes == sorted(sizes, reverse=True)
 
 
 # ---- single-split steps: the split kernel writes the output itself, no combine launch

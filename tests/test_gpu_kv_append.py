@@ -315,7 +315,7 @@ def test_append_also_ranks_sequences(fd):
     real = fd.kernels.kv_append._decode
 
     def spy(*a, **kw):
-        seen["order"], seen["lens"] = kw.get("seq_order"), kw.get("seq_order_lens")
+        seen["order"], seen["lens"], seen["items"] = kw.get("seq_order"), kw.get("seq_order_lens"), kw.get("item_order")
         return real(*a, **kw)
     fd.kernels.kv_append._decode = spy
     try:
@@ -324,9 +324,18 @@ def test_append_also_ranks_sequences(fd):
     finally:
         fd.kernels.kv_append._decode = real
     torch.cuda.synchronize()
-    assert seen["order"] is not None
-    assert seen["order"].cpu().tolist() == sorted(range(B), key=lambda i: (-int(new_lens[i]), i))
-    assert seen["lens"].cpu().tolist() == sorted(new_lens.tolist(), reverse=True)
+    if seen["items"] is not None:
+        # the append launch computed the decode's (sequence, range) issue order: every pair once, with the grown
+        # length of its sequence beside it
+        it = seen["items"].cpu().view(2, -1)
+        S = it.shape[1] // B
+        seqs, ranges = (it[0] & 0xFFFF).tolist(), ((it[0] >> 16) & 0xFFFF).tolist()
+        assert sorted(zip(seqs, ranges)) == [(b, r) for b in range(B) for r in range(S)]
+        assert it[1].tolist() == [int(new_lens[b]) for b in seqs]
+    else:
+        assert seen["order"] is not None
+        assert seen["order"].cpu().tolist() == sorted(range(B), key=lambda i: (-int(new_lens[i]), i))
+        assert seen["lens"].cpu().tolist() == sorted(new_lens.tolist(), reverse=True)
     assert_out_close(out[:, 0], ref)
 
 

@@ -213,6 +213,18 @@ def test_split_plan_policy(fd):
     assert plan(1, 96, 12, 128, 1 << 20, P=1) == 128
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1
+    # the part of the plan that fills the chip, without the bound on the length of a split: what a sequence gets
+    # however short it is (fd_params.split_adapt)
+    def fill(B, Hq, Hkv, S, max_pages, P=16, kv=L.FD_BF16, D=128):
+        p = L.FdParams()
+        p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits = Hq, Hkv, D, P, S
+        p.num_pages, p.max_pages_per_seq, p.q_dtype, p.kv_dtype = 1 << 20, max_pages, L.FD_BF16, kv
+        return lib.fd_plan_min_splits(ctypes.byref(p), B)
+    assert fill(8, 32, 8, 32, 512) == 8 and fill(8, 32, 8, 32, 8192) == 8      # config 2, whatever the table's width
+    assert plan(8, 32, 8, 32, 8192) == 32                                      # ... while the grid covers the capacity
+    assert fill(64, 32, 8, 32, 8192) == 1 and plan(64, 32, 8, 32, 8192) == 32  # a batch fills the chip by itself
+    assert fill(1, 8, 1, 256, 65536) == 256
+    assert fill(0, 32, 8, 32, 512) < 0 and lib.fd_plan_min_splits(None, 1) < 0
     for args in [(3, 16, 16, 32, 83), (7, 6, 1, 5, 1000), (2, 64, 8, 64, 100000)]:
         got = plan(*args)
         assert 1 <= got <= args[3]

@@ -24,7 +24,8 @@ FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_plan_splits", "fd_kv_append",
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
+                    "fd_kv_append",
                     "fd_last_error", "fd_abi_version")
 
 _DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
@@ -51,6 +52,8 @@ class FdParams(Structure):
         ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
         ("path", c_int32), ("waves_per_block", c_int32), ("seq_order_lens", c_void_p),
         ("split_align", c_int32),
+        ("split_adapt", c_int32),
+        ("seq_order_items", c_int32),
     ]
 
 
@@ -97,8 +100,12 @@ def load_library(path: str = None) -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
         c_int32, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p,
         c_int32, c_void_p, POINTER(FdParams)]
+    lib.fd_schedule_items.restype = c_int32
+    lib.fd_schedule_items.argtypes = [c_void_p, c_void_p, c_int32, c_void_p, POINTER(FdParams)]
     lib.fd_plan_splits.restype = c_int32
     lib.fd_plan_splits.argtypes = [POINTER(FdParams), c_int32]
+    lib.fd_plan_min_splits.restype = c_int32
+    lib.fd_plan_min_splits.argtypes = [POINTER(FdParams), c_int32]
     lib.fd_kv_append.restype = c_int32
     lib.fd_kv_append.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,

@@ -60,6 +60,17 @@ int mfma_head_block(int head_dim, int group, int kv_dtype) {
   return (group > 16 && head_dim == 128 && kv16) ? 32 : 16;
 }
 
+// fd_params.split_adapt: 0, or a power of two together with a split alignment and a power-of-two split count.
+int check_split_adapt(const char* fn, const fd_params* p) {
+  const int k = p->split_adapt;
+  if (k == 0) return FD_OK;
+  if (k < 0 || (k & (k - 1)) || p->split_align <= 0 || (p->num_splits & (p->num_splits - 1)))
+    return fail(FD_ERR_INVALID_ARG,
+                "%s: split_adapt %d needs a power of two, split_align > 0 and a power-of-two num_splits (%d)", fn, k,
+                p->num_splits);
+  return FD_OK;
+}
+
 // Launch-shape policy, from sweeps on one MI355X (256 CUs): the MFMA kernels stream best with about
 // 1024 waves in flight (16 KB of loads each), the VALU kernel with about 2048 (8 KB each), each walking
 // a long token range (every wave pays a fixed prologue / epilogue, and every split adds a partial for
@@ -67,7 +78,7 @@ int mfma_head_block(int head_dim, int group, int kv_dtype) {
 constexpr int64_t kTargetWaves = 1024;
 constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
-constexpr int64_t kMaxTokensPerSplit = 4096;   // keeps a ragged batch balanceable by the dispatcher
+constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
 
 // Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
 // split) where the caller leaves the choice to the library) and FD_HEADS_PER_BLOCK (members per workgroup).
@@ -132,7 +143,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
                const int32_t* kv_lens, int32_t batch, int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok,
                int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
                int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p,
-               const FusedTail* tail, bool* fused, bool no_lse = false) {
+               const FusedTail* tail, bool* fused, bool no_lse = false, bool skip_empty = false) {
   if (fused) *fused = false;
   if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (!q || !k_cache || !v_cache || !out_split || !block_table || !kv_lens)
@@ -167,16 +178,22 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
       stride_v_tok * kvsz >= ((int64_t)1 << 31))
     return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
   const int G = p->q_heads / p->kv_heads;
-  const int64_t max_tok_split = ((int64_t)p->max_pages_per_seq * p->page_size + p->num_splits - 1) / p->num_splits;
+  int64_t max_tok_split = ((int64_t)p->max_pages_per_seq * p->page_size + p->num_splits - 1) / p->num_splits;
+  if (p->split_adapt > 0 && max_tok_split < kMinTokensPerRange)   // ranges by each sequence's own length
+    max_tok_split = kMinTokensPerRange;
 
   SplitArgs a;
   memset(&a, 0, sizeof(a));
   a.q = q; a.k = k_cache; a.v = v_cache; a.out = out_split; a.lse = lse_split;
   a.bt = block_table; a.kv_lens = kv_lens; a.order = seq_order; a.order_lens = seq_order ? p->seq_order_lens : nullptr;
+  if (seq_order && p->seq_order_items) {   // (sequence, range) items and, behind them, their lengths
+    a.order_items = 1;
+    a.order_lens = seq_order + (int64_t)batch * p->num_splits;
+  }
   a.k_scale = p->k_scale; a.v_scale = p->v_scale;
   a.sq_b = stride_q_bs; a.sq_h = stride_q_h; a.sk_t = stride_k_tok; a.sk_h = stride_k_h;
   a.sv_t = stride_v_tok; a.sv_h = stride_v_h; a.so_b = stride_o_bs; a.so_h = stride_o_h; a.so_s = stride_o_split;
-  a.sbt = stride_table_bs; a.no_lse = no_lse ? 1 : 0;
+  a.sbt = stride_table_bs; a.no_lse = no_lse ? 1 : 0; a.skip_empty = skip_empty ? 1 : 0;
   a.sm_scale = sm_scale; a.soft_cap = p->soft_cap > 0.f ? p->soft_cap : 0.f;
   a.batch = batch; a.Hq = p->q_heads; a.Hkv = p->kv_heads; a.G = G; a.S = p->num_splits; a.P = p->page_size;
   div_magic((uint32_t)p->page_size, &a.div_magic, &a.div_shift);
@@ -184,6 +201,8 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
     return fail(FD_ERR_INVALID_ARG, "%s: split_align %d (0 or a power of two <= 4096)", fn, p->split_align);
   a.per_mask = p->split_align ? p->split_align - 1 : 0;
+  if (int rc = check_split_adapt(fn, p)) return rc;
+  a.adapt = p->split_adapt;
   a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
   a.q_dtype = p->q_dtype; a.mid_dtype = p->mid_dtype;
   a.vec_out = (p->mid_dtype == FD_F32 && aligned16(out_split) && stride_o_bs % 4 == 0 && stride_o_h % 4 == 0 &&
@@ -216,7 +235,10 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   }
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
-  const int64_t wgs = (int64_t)batch * a.S * a.Hkv * a.nhb;
+  // Ranges that are certain to be busy per sequence: all of them, or, when the ranges follow each sequence's own
+  // length, only the ones every sequence gets (the rest of the grid may be empty ranges).
+  const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : a.S;
+  const int64_t wgs = (int64_t)batch * busy_splits * a.Hkv * a.nhb;
   // the two-block MFMA kernel needs the register file of a whole SIMD per wave: workgroups of at most 4 waves
   const int max_waves = use_mfma && a.hbsz > 16 ? 4 : 8;
   int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
@@ -277,6 +299,20 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
 extern "C" {
 
+// The ranges of a decode step with these parameters, for the schedulers.
+static int range_plan(const char* fn, const fd_params* p, RangePlan* rp) {
+  if (p->num_splits <= 0 || p->num_splits > 65535)
+    return fail(FD_ERR_INVALID_ARG, "%s: num_splits %d", fn, p->num_splits);
+  if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
+    return fail(FD_ERR_INVALID_ARG, "%s: split_align %d (0 or a power of two <= 4096)", fn, p->split_align);
+  if (int rc = check_split_adapt(fn, p)) return rc;
+  rp->S = p->num_splits;
+  div_magic((uint32_t)p->num_splits, &rp->s_magic, &rp->s_shift);
+  rp->per_mask = p->split_align ? p->split_align - 1 : 0;
+  rp->adapt = p->split_adapt;
+  return FD_OK;
+}
+
 static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, void* out, float* lse_out,
                         const int32_t* seqlens, int32_t batch, int32_t q_heads, int32_t num_partials,
                         int64_t stride_mid_ob, int64_t stride_mid_oh, int64_t stride_mid_os, int64_t stride_obs,
@@ -328,27 +364,33 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
   tail.extra_lse = extra_lse; tail.stride_obs = stride_obs; tail.stride_oh = stride_oh; tail.num_extra = num_extra;
   tail.lse_column = combine_mode == FD_COMBINE_SPLIT_LSE;
   bool fused = false;
+  // Ranges that follow each sequence's own length leave most slots of a long split list empty: beyond what the
+  // small combine kernel takes in one gulp, the empty ranges' workgroups write nothing and the combine derives
+  // from kv_lens which slots hold a partial (one more dependent load there, no traffic for the empty ones).
+  const bool skip_empty = p && p->split_adapt > 0 && p->num_splits > kCombineSmallMax && !tickets;
   int rc = split_impl("fd_decode", stream, q, k_cache, v_cache, out_split, lse_split, sm_scale, block_table, kv_lens,
                       batch, stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_o_bs,
-                      stride_o_h, stride_o_split, stride_table_bs, seq_order, p, &tail, &fused);
+                      stride_o_h, stride_o_split, stride_table_bs, seq_order, p, &tail, &fused, false, skip_empty);
   if (rc != FD_OK || fused || batch == 0) return rc;
   return combine_impl(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
                       stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out,
-                      extra_lse, num_extra, p, true);
+                      extra_lse, num_extra, p, !skip_empty);
 }
 
-int fd_plan_splits(const fd_params* p, int32_t batch) {
-  if (!p) return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: params is NULL");
+// Splits a shape needs to fill the chip, regardless of how long its sequences are (a power of two >= 1), or a
+// negative fd_status.  fd_plan_splits adds the bound on the length of a split and the caller's limit.
+static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batch) {
+  if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (batch <= 0 || p->q_heads <= 0 || p->kv_heads <= 0 || p->q_heads % p->kv_heads != 0 || p->num_splits <= 0 ||
       p->page_size <= 0 || p->max_pages_per_seq <= 0)
-    return fail(FD_ERR_INVALID_ARG, "fd_plan_splits: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0");
+    return fail(FD_ERR_INVALID_ARG, "%s: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0", fn);
   const int G = p->q_heads / p->kv_heads;
   const bool mfma = mfma_shape_ok(p->head_dim, G, p->kv_dtype) && p->path != FD_PATH_VALU;
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
-  int64_t s;
+  int64_t s = 1;
   if (mfma) {
     // (1) one workgroup per CU at the full member width (sibling KV heads, or head blocks of one KV head): measured
     // over head dims, cache dtypes and batch sizes, 256 workgroups x 4 waves beats 512 x 2 and 128 x 8 ...
@@ -361,7 +403,6 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
       members = row_bytes > 0 && row_bytes < 512 ? 512 / row_bytes : 1;
       while (members > 1 && p->kv_heads % members != 0) members >>= 1;
     }
-    s = 1;
     while (s * groups < kMinWorkgroups * members) s <<= 1;
     // (2) ... and a whole number of workgroups per CU, or at least four, while a split of a full-length sequence
     // keeps 512 tokens: equal work items run in one round, and 1.5 workgroups per CU take as long as 2
@@ -370,11 +411,22 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
       s <<= 1;
   } else {
     // the VALU kernel keeps half as many bytes in flight per wave: twice the waves, four per (KV head, split)
-    s = 1;
     while (s * 4 * groups < kTargetWavesValu) s <<= 1;
   }
+  return s;
+}
+
+int fd_plan_min_splits(const fd_params* p, int32_t batch) {
+  const int64_t s = plan_fill_splits("fd_plan_min_splits", p, batch);
+  return (int)(s > 65536 ? 65536 : s);
+}
+
+int fd_plan_splits(const fd_params* p, int32_t batch) {
+  int64_t s = plan_fill_splits("fd_plan_splits", p, batch);
+  if (s < 0) return (int)s;
   // (3) in a batch, enough splits that no split of a full-length sequence is longer than kMaxTokensPerSplit: the
   // dispatcher evens out ragged lengths with them
+  const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
   if (batch > 1) {
     while (s * kMaxTokensPerSplit < max_tokens) s <<= 1;
   }
@@ -419,6 +471,14 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
     return fail(FD_ERR_INVALID_ARG, "fd_combine: split_align %d (0 or a power of two <= 4096)", p->split_align);
   a.per_mask = p->split_align ? p->split_align - 1 : 0;
+  if (mode != FD_COMBINE_RANK) {
+    a.adapt = p->split_adapt;
+    if (a.adapt < 0 || (a.adapt & (a.adapt - 1)) || (a.adapt > 0 && (p->split_align <= 0 || (num_partials & (num_partials - 1)))))
+      return fail(FD_ERR_INVALID_ARG,
+                  "fd_combine: split_adapt %d needs a power of two, split_align > 0 and a power-of-two num_partials (%d)",
+                  a.adapt, num_partials);
+  }
+  div_magic((uint32_t)num_partials, &a.s_magic, &a.s_shift);
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;
@@ -486,7 +546,14 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
       return fail(FD_ERR_ALIGNMENT, "%s: k_new / v_new rows must be 16-byte aligned (pointer and strides)", fn);
     if (stride_k_tok <= 0 || stride_v_tok <= 0) return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
     a.k_new = k_new; a.v_new = v_new; a.k_cache = k_cache; a.v_cache = v_cache;
-    a.bt = block_table; a.kv_lens = kv_lens; a.kv_lens_out = kv_lens_out; a.seq_order = seq_order_out;
+    a.bt = block_table; a.kv_lens = kv_lens; a.kv_lens_out = kv_lens_out;
+    if (seq_order_out && p->seq_order_items) {
+      if (batch > 256) return fail(FD_ERR_TOO_LARGE, "%s: work-item order with batch %d > 256 (use fd_schedule_items)", fn, batch);
+      if (int rc = range_plan(fn, p, &a.ranges)) return rc;
+      a.items = seq_order_out;
+    } else {
+      a.seq_order = seq_order_out;
+    }
     a.k_scale = p->k_scale; a.v_scale = p->v_scale;
     a.skn_b = stride_kn_b; a.skn_t = stride_kn_t; a.skn_h = stride_kn_h;
     a.svn_b = stride_vn_b; a.svn_t = stride_vn_t; a.svn_h = stride_vn_h;
@@ -528,6 +595,23 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
   if (rc == FD_ERR_LAUNCH) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
   if (rc == FD_ERR_TOO_LARGE) return fail(rc, "%s: batch * new_tokens * heads too large for one launch", fn);
   if (rc != FD_OK) return fail(rc, "%s: no kernel for q_dtype %d -> kv_dtype %d", fn, p->q_dtype, kv_dtype);
+  return FD_OK;
+}
+
+int fd_schedule_items(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* item_order, const fd_params* p) {
+  const char* fn = "fd_schedule_items";
+  if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
+  if (!kv_lens || !item_order) return fail(FD_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+  if (batch < 0) return fail(FD_ERR_INVALID_ARG, "%s: batch = %d", fn, batch);
+  if (batch == 0) return FD_OK;
+  if (batch > kMaxItemBatch) return fail(FD_ERR_TOO_LARGE, "%s: batch %d > %d (use fd_schedule)", fn, batch, kMaxItemBatch);
+  if (p->page_size <= 0 || p->max_pages_per_seq <= 0)
+    return fail(FD_ERR_INVALID_ARG, "%s: page_size / max_pages_per_seq must be > 0", fn);
+  RangePlan rp;
+  if (int rc = range_plan(fn, p, &rp)) return rc;
+  int rc = fd_launch_schedule_items((hipStream_t)stream, kv_lens, batch, (int64_t)p->max_pages_per_seq * p->page_size, rp,
+                                    item_order);
+  if (rc != FD_OK) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
   return FD_OK;
 }
 

@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   int kv_len = 0, per = 0;
   if (a.mode != FD_COMBINE_RANK && !own) {
     kv_len = max(a.seqlens[b], 0);
-    per = ((kv_len + S - 1) / S + a.per_mask) & ~a.per_mask;
+    per = tokens_per_range(kv_len, S, a.s_magic, a.s_shift, a.per_mask, a.adapt);
   }
   // LSE of partial s, -inf when the partial is not valid
   auto partial_lse = [&](int s) -> float {
@@ -160,7 +160,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
 // same call: every slot is written (an empty split holds out = 0, lse = -inf), so validity needs no
 // kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which leaves one
 // dependent memory round trip.  Thread (r, c): partial r (and r + ROWS), 128-bit column chunk c.
-constexpr int kSmallMax = 16;
+constexpr int kSmallMax = kCombineSmallMax;
 
 template <int D>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_small_kernel(const CombineArgs a) {
@@ -235,6 +235,19 @@ __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restr
   order[rank] = i;
 }
 
+// One workgroup: the (sequence, range) issue order of a decode step (fd_schedule_items_block).
+__global__ void __launch_bounds__(kMaxItemBatch) fd_schedule_items_kernel(const int32_t* __restrict__ kv_lens, int batch,
+                                                                        int64_t capacity, RangePlan ranges,
+                                                                        int32_t* __restrict__ items) {
+  __shared__ uint64_t s_key[kMaxItemBatch];
+  __shared__ int32_t s_n[kMaxItemBatch];
+  auto len_of = [&](int j) {
+    const int64_t len = kv_lens[j];
+    return (int)(len < 0 ? 0 : (len > capacity ? capacity : len));   // as the split kernels clamp it
+  };
+  fd_schedule_items_block(threadIdx.x, blockDim.x, batch, len_of, ranges, items, s_key, s_n);
+}
+
 }  // namespace
 
 int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
@@ -266,5 +279,13 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
 int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, int32_t* order) {
   const unsigned grid = (unsigned)((batch + 255) / 256);
   hipLaunchKernelGGL(fd_schedule_kernel, dim3(grid), dim3(256), 0, stream, kv_lens, batch, order);
+  return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
+}
+
+int fd_launch_schedule_items(hipStream_t stream, const int32_t* kv_lens, int batch, int64_t capacity,
+                             const RangePlan& ranges, int32_t* items) {
+  if (batch > kMaxItemBatch) return FD_ERR_TOO_LARGE;
+  const unsigned threads = (unsigned)((batch + 63) / 64 * 64);
+  hipLaunchKernelGGL(fd_schedule_items_kernel, dim3(1), dim3(threads), 0, stream, kv_lens, batch, capacity, ranges, items);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }

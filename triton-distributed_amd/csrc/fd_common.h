@@ -33,6 +33,7 @@ struct SplitArgs {
   const int32_t* kv_lens;
   const int32_t* order;  // nullptr: identity
   const int32_t* order_lens;  // nullptr, or kv_lens[order[r]] at index r
+  int32_t order_items;   // 1: order holds batch * S work items (sequence | range << 16), order_lens their lengths
   const float* k_scale;
   const float* v_scale;
   int64_t sq_b, sq_h, sk_t, sk_h, sv_t, sv_h, so_b, so_h, so_s, sbt;
@@ -52,6 +53,8 @@ struct SplitArgs {
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
   int32_t per_mask;               // split_align - 1 (0: the reference's ranges): tokens per split are rounded up
+  int32_t adapt;                  // fd_params.split_adapt: ranges per sequence by its own length (0: always S)
+  int32_t skip_empty;             // 1: a workgroup whose range is empty writes nothing (the combine knows the ranges)
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
   int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
@@ -76,8 +79,17 @@ struct CombineArgs {
   int32_t vec_mid;  // 1: every mid_o row start is 16-byte aligned (128-bit loads allowed)
   int32_t cg_shift; // log2 of the 128-bit column groups a workgroup of the general kernel covers (set by the launcher)
   int32_t per_mask;           // as SplitArgs::per_mask, for the validity of split ranges
+  int32_t adapt;              // as SplitArgs::adapt
+  uint32_t s_magic, s_shift;  // n / num_partials, as in SplitArgs
   int32_t all_slots_written;  // 1: the partials come from this library's split kernel in the same call, which
                               // writes every slot (empty splits as out = 0, lse = -inf)
+};
+
+// How a decode step cuts a sequence into ranges: what the scheduler needs to know of it.
+struct RangePlan {
+  int32_t S;                  // ranges per sequence (grid slots)
+  uint32_t s_magic, s_shift;  // n / S
+  int32_t per_mask, adapt;    // as in SplitArgs
 };
 
 // Arguments of the KV-append / rotary kernel.
@@ -89,7 +101,9 @@ struct AppendArgs {
   const int32_t* bt;
   const int32_t* kv_lens;
   int32_t* kv_lens_out;  // nullptr or [batch]
-  int32_t* seq_order;    // nullptr or [batch]: sequences ranked by grown length, longest first
+  int32_t* seq_order;    // nullptr or [2 * batch]: sequences ranked by grown length, longest first, then those lengths
+  int32_t* items;        // nullptr or [2 * batch * ranges.S]: work items of the decode that follows (fd_schedule_items)
+  RangePlan ranges;      // how that decode cuts a sequence into ranges (items only)
   int32_t data_blocks;   // workgroups that move data; the ones after them compute seq_order
   const float* k_scale;
   const float* v_scale;
@@ -177,7 +191,7 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
   FD_PIN(sq_b); FD_PIN(sq_h); FD_PIN(sk_t); FD_PIN(sk_h); FD_PIN(sv_t); FD_PIN(sv_h); FD_PIN(sbt);
   FD_PIN(sm_scale); FD_PIN(batch); FD_PIN(G); FD_PIN(S); FD_PIN(P); FD_PIN(max_pages); FD_PIN(num_pages);
   FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(member_hb); FD_PIN(s_magic);
-  FD_PIN(s_shift); FD_PIN(per_mask);
+  FD_PIN(s_shift); FD_PIN(per_mask); FD_PIN(adapt); FD_PIN(skip_empty); FD_PIN(order_items);
   // what the epilogue reads, so that it does not wait for the argument segment either
   FD_PIN(out); FD_PIN(lse); FD_PIN(so_b); FD_PIN(so_h); FD_PIN(so_s); FD_PIN(tickets); FD_PIN(mid_dtype);
   FD_PIN(vec_out); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
@@ -189,9 +203,48 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
 // split.  Sibling waves therefore request neighbouring 128/256-byte pieces of the same token rows
 // from the same CU at about the same time, which the memory system serves markedly better than the
 // same pieces requested by workgroups on different XCDs (measured with a pure-read probe: 5.3 vs
-// 5.85-6.1 TB/s for 128-byte rows).  blockIdx.z is the rank of the sequence in the issue order.
+// 5.85-6.1 TB/s for 128-byte rows).
+//
+// Issue order (workgroups are issued x-fastest and handed to the 8 XCDs, and within an XCD to its CUs, round-robin):
+//  * every sequence uses all S ranges (the reference's rule): grid (x, S, batch), z = rank of the sequence -- with a
+//    ranked batch the largest items are issued first and the smallest last;
+//  * ranges by each sequence's own length, unscheduled: grid (x, batch, S) -- the split is the slowest dimension, so the
+//    ranges every sequence has come first as one contiguous run and the empty ones last.  Next to x, the busy
+//    workgroups of sequences that use only their first range would all fall on the same XCDs (measured: half the chip
+//    idle, 73 instead of 43 us for 64 sequences of 1000 tokens with S = 2); rotating the split by the rank spreads the
+//    XCDs but alternates busy and empty workgroups over the CUs of an XCD (57 us);
+//  * scheduled (order_items): the issue order is a list of (sequence, range) items, non-empty ranges first, largest
+//    first, empty ones last (fd_schedule_items_block).
+
+// Most partials the small combine kernel takes (one dependent round trip, every slot must hold a partial).
+constexpr int kCombineSmallMax = 16;
+
+// Ranges by each sequence's own length (split_adapt): a range is not made shorter than this unless the
+// sequence would otherwise get fewer ranges than the shape needs to fill the chip.
+constexpr int kMinTokensPerRange = 1024;
+// A batch gets enough splits that no range of a full-length sequence is longer than this (the split plan).
+constexpr int kMaxTokensPerRange = 4096;
+
+// Tokens per split range of a sequence of kv_len tokens.  Reference rule: ceil(kv_len / S) (flash_decode.py:193-195).
+// With adapt > 0 (a power of two, the ranges every sequence needs so that the batch fills the chip) a short
+// sequence is not cut into S slivers: per = max(ceil(kv_len / S), min(ceil(kv_len / adapt), 1024)), i.e. adapt
+// ranges up to adapt * 1024 tokens, 1024-token ranges up to S * 1024 tokens, S ranges beyond.  per_mask rounds the
+// result up to the split alignment.  The split kernels and the combine kernel both call this, so they agree on
+// which ranges are empty.
+__device__ __forceinline__ int tokens_per_range(int kv_len, int S, uint32_t s_magic, uint32_t s_shift, int per_mask,
+                                                int adapt) {
+  // ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)
+  int per = (int)(((uint64_t)(uint32_t)(kv_len + S - 1) * s_magic) >> s_shift);
+  if (adapt > 0) {
+    const int floor_ranges = (kv_len + adapt - 1) >> (31 - __clz(adapt));   // ceil(kv_len / adapt)
+    per = max(per, min(floor_ranges, kMinTokensPerRange));
+  }
+  return (per + per_mask) & ~per_mask;
+}
+
 struct WorkItem {
   int b, s, kvh, hb, start, end;
+  bool skip;  // empty range and nothing to write: the workgroup may leave at once (uniform over the workgroup)
   int kvh0;   // first KV head of the workgroup
   int hb0;    // first head block of the workgroup
   int sub;    // token sub-range index of this wave
@@ -202,10 +255,25 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   WorkItem w;
   // The sequence and its length first: these scalar loads head the chain length -> block table -> K/V rows that
   // every wave has to walk before it can stream.
-  const int r = blockIdx.z;
-  int b = a.order ? a.order[r] : r;
-  w.b = min(max(b, 0), a.batch - 1);
-  int64_t len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
+  int b, s;
+  int64_t len;
+  if (a.order_items) {
+    // scheduled: item k of the issue order names its sequence and range (grid (x, S, batch), y fastest)
+    const int k = blockIdx.y + a.S * blockIdx.z;
+    const uint32_t item = (uint32_t)a.order[k];
+    len = a.order_lens[k];
+    b = item & 0xffffu;
+    s = item >> 16;
+    w.b = min(b, a.batch - 1);
+  } else {
+    // ranges by each sequence's own length: grid (x, batch, S), else grid (x, S, batch)
+    const bool slab_major = a.adapt > 0;
+    const int r = slab_major ? blockIdx.y : blockIdx.z;
+    s = slab_major ? blockIdx.z : blockIdx.y;
+    b = a.order ? a.order[r] : r;
+    w.b = min(max(b, 0), a.batch - 1);
+    len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
+  }
   fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
 
   const int wave = threadIdx.x >> 6;
@@ -241,17 +309,16 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     }
     w.nsub = a.nsub;
   }
-  w.s = blockIdx.y;
+  w.s = min(s, a.S - 1);
   int64_t cap = (int64_t)a.max_pages * a.P;
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
-  // per = ceil(kv_len / S) by multiplication (kv_len + S - 1 < 2^31 is checked on the host)
-  int per = (int)(((uint64_t)(uint32_t)(kv_len + a.S - 1) * a.s_magic) >> a.s_shift);
-  per = (per + a.per_mask) & ~a.per_mask;
+  const int per = tokens_per_range(kv_len, a.S, a.s_magic, a.s_shift, a.per_mask, a.adapt);
   int64_t st = (int64_t)per * w.s;
   w.start = st > kv_len ? kv_len : (int)st;
   int64_t en = st + per;
   w.end = en > kv_len ? kv_len : (int)en;
+  w.skip = a.skip_empty && w.start >= w.end;
   return w;
 }
 
@@ -429,6 +496,60 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
   }
 }
 
+// Sequences one scheduling workgroup ranks (its LDS holds 12 bytes per sequence).
+constexpr int kMaxItemBatch = 1024;
+
+// Work-item order for the split kernels, computed by ONE workgroup of nthreads threads (batch <= kMaxItemBatch).
+// items[k], k < batch * S, = sequence | range << 16: first the non-empty ranges, sequence by sequence in descending
+// (tokens per range, length) order, ties by index -- all ranges of a sequence have the same size, so this is
+// largest-item-first -- then the empty ranges.  items[batch * S + k] = the length of item k's sequence.
+// len_of(j) = length of sequence j as the decode will see it.  s_key / s_n: LDS, batch entries each.
+template <typename LenFn>
+__device__ __forceinline__ void fd_schedule_items_block(int tid, int nthreads, int batch, LenFn len_of,
+                                                        const RangePlan& rp, int32_t* items, uint64_t* s_key,
+                                                        int32_t* s_n) {
+  for (int j = tid; j < batch; j += nthreads) {
+    const int len = len_of(j);
+    const int per = tokens_per_range(len, rp.S, rp.s_magic, rp.s_shift, rp.per_mask, rp.adapt);
+    int n = 0;
+    if (len > 0) {   // n = ceil(len / per) <= S without an integer division
+      n = (int)((float)len / (float)per);
+      while ((int64_t)n * per < len) ++n;
+      while (n > 0 && (int64_t)(n - 1) * per >= len) --n;
+    }
+    s_key[j] = ((uint64_t)(uint32_t)per << 32) | (uint32_t)len;
+    s_n[j] = n;
+  }
+  __syncthreads();
+  const int total = batch * rp.S;
+  for (int i = tid; i < batch; i += nthreads) {
+    const uint64_t mine = s_key[i];
+    int rank = 0, off = 0, active = 0;
+    for (int j = 0; j < batch; ++j) {
+      const uint64_t other = s_key[j];
+      const int n = s_n[j];
+      const bool before = other > mine || (other == mine && j < i);
+      rank += before ? 1 : 0;
+      off += before ? n : 0;
+      active += n;
+    }
+    const int n_i = s_n[i];
+    const int len_i = (int)(uint32_t)mine;
+    const int empty0 = active + rank * rp.S - off;   // the empty ranges of the sequences before this one
+    for (int t = 0; t < rp.S; ++t) {
+      const int k = t < n_i ? off + t : empty0 + (t - n_i);
+      items[k] = (int32_t)((uint32_t)i | ((uint32_t)t << 16));
+      items[total + k] = len_i;
+    }
+  }
+}
+
+// Launch grid of the split kernels (see decode_work_item).
+inline dim3 fd_split_grid(const SplitArgs& a) {
+  if (a.adapt > 0 && !a.order_items) return dim3((unsigned)a.grid_x, (unsigned)a.batch, (unsigned)a.S);
+  return dim3((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
+}
+
 // Launchers implemented in the kernel translation units (host side).
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap);
 int fd_launch_split_mfma_d64(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap);
@@ -438,4 +559,6 @@ int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype
 int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int waves);
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a);
 int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, int32_t* order);
+int fd_launch_schedule_items(hipStream_t stream, const int32_t* kv_lens, int batch, int64_t capacity,
+                             const RangePlan& ranges, int32_t* items);
 int fd_launch_kv_append(hipStream_t stream, const AppendArgs& a, int src_dtype, int kv_dtype);

@@ -124,15 +124,23 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
   const int heads = hq + 2 * hkv;               // rows per (sequence, token): K heads, V heads, Q heads
   if ((int)blockIdx.x >= a.data_blocks) {
     // Trailing workgroups: issue order for the decode that follows (same ranking as the stand-alone
-    // scheduler: grown length descending, ties by index), so that it costs no launch of its own.
-    const int i = ((int)blockIdx.x - a.data_blocks) * blockDim.x + threadIdx.x;
-    if (i >= a.batch) return;
+    // schedulers), so that it costs no launch of its own.
     const int64_t cap = (int64_t)a.max_pages * a.P;
     auto grown = [&](int b) {
       int64_t len = a.kv_lens[b];
       len = (len < 0 ? 0 : len) + a.T;
       return len > cap ? cap : len;
     };
+    if (a.items) {   // one workgroup: (sequence, range) items, batch <= 256
+      __shared__ uint64_t s_key[256];
+      __shared__ int32_t s_n[256];
+      fd_schedule_items_block(threadIdx.x, blockDim.x, a.batch, [&](int b) { return (int)grown(b); }, a.ranges,
+                              a.items, s_key, s_n);
+      return;
+    }
+    // per-sequence order: grown length descending, ties by index
+    const int i = ((int)blockIdx.x - a.data_blocks) * blockDim.x + threadIdx.x;
+    if (i >= a.batch) return;
     const int64_t mine = grown(i);
     int rank = 0;
     for (int j = 0; j < a.batch; ++j) {
@@ -234,7 +242,12 @@ int fd_launch_kv_append(hipStream_t stream, const AppendArgs& args, int src_dtyp
   int64_t blocks = (threads + 255) / 256;
   if (blocks > 0x7fff0000LL) return FD_ERR_TOO_LARGE;
   a.data_blocks = (int32_t)blocks;
-  if (a.seq_order) blocks += (a.batch + 255) / 256;
+  if (a.items) {
+    if (a.batch > 256) return FD_ERR_TOO_LARGE;
+    blocks += 1;
+  } else if (a.seq_order) {
+    blocks += (a.batch + 255) / 256;
+  }
   const dim3 grid((unsigned)blocks);
   switch (src_dtype) {
     case FD_F32: return launch_src<float>(stream, a, kv_dtype, grid);

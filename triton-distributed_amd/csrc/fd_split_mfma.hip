@@ -61,6 +61,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
   const int c = lane & 15;
 
   const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
+  if (w.skip) return;   // empty range, and the combine does not expect a partial from it
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
   const int tpw = (ntiles + w.nsub - 1) / w.nsub;
@@ -296,7 +297,7 @@ static auto pick_kernel(bool soft_cap, int nb) -> void (*)(const SplitArgs) {
 
 // a.hbsz = query heads per head block: up to 16 (one MFMA column block per wave) or 32 (two)
 int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
-  const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid = fd_split_grid(a);
   const unsigned block = 64u * waves;
   const int nb = a.hbsz > 16 ? 2 : 1;
   size_t lds = (size_t)waves * wave_lds(nb);

@@ -50,6 +50,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
   const int c = lane & 15;
 
   const WorkItem w = decode_work_item(a);
+  if (w.skip) return;   // empty range, and the combine does not expect a partial from it
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
   const int tpw = (ntiles + w.nsub - 1) / w.nsub;
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
 }  // namespace
 
 int fd_launch_split_mfma_d256(hipStream_t stream, const SplitArgs& a, int kv_dtype, int waves, bool soft_cap) {
-  const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid = fd_split_grid(a);
   const unsigned block = 64u * waves;
   size_t lds = (size_t)waves * kWaveLds;
   if (a.tickets) {

@@ -88,6 +88,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   const int c = lane % LPR;           // chunk of the row
 
   const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
+  if (w.skip) return;   // empty range, and the combine does not expect a partial from it
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + TILE - 1) / TILE : 0;
   const int tpw = (ntiles + w.nsub - 1) / w.nsub;
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 
 template <int KV, int D>
 int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
-  const dim3 grid((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
+  const dim3 grid = fd_split_grid(a);
   const unsigned block = 64u * waves;
   void (*kern)(const SplitArgs) = nullptr;
   int gh = a.hbsz;

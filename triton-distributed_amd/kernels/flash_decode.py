@@ -98,7 +98,7 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 
 
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
-                 waves_per_block, seq_order_lens=None, split_align=0) -> FdParams:
+                 waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0) -> FdParams:
     p = FdParams()
     p.q_heads = q.shape[1]
     p.kv_heads = k_cache.shape[2]
@@ -118,12 +118,45 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
     p.waves_per_block = waves_per_block
     p.seq_order_lens = seq_order_lens.data_ptr() if seq_order_lens is not None else None
     p.split_align = split_align
+    p.split_adapt = split_adapt
+    p.seq_order_items = seq_order_items
     return p
+
+
+MAX_ITEM_BATCH = 1024       # sequences fd_schedule_items ranks in one launch
+MAX_FUSED_ITEM_BATCH = 256  # ... and fd_kv_append in its trailing workgroup
+
+
+def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=None, path="auto", waves_per_block=0):
+    """The split plan of a decode step whose partials stay inside the library: ``(num_splits, split_adapt)`` --
+    grid slots per sequence and the ranges every sequence gets however short it is (``fd_plan_splits``,
+    ``fd_plan_min_splits``; cached by shape).  ``kv_split`` is the caller's bound, -1 leaves it to the library."""
+    batch, q_heads, q_head_dim = q.shape
+    page_size, kv_heads = k_cache.shape[1], k_cache.shape[2]
+    bound = auto_split_bound(block_table.shape[1] * page_size) if kv_split == -1 else kv_split
+    key = (batch, q_heads, kv_heads, q_head_dim, page_size, bound, block_table.shape[1], k_cache.dtype,
+           k_scale is not None, path)
+    planned = _PLAN_CACHE.get(key)
+    if planned is None:
+        lib = load_library()
+        plan = _make_params(q, k_cache, block_table, bound, 0.0, FD_F32, FD_F32, k_scale, v_scale, path,
+                            waves_per_block)
+        planned = (lib.fd_plan_splits(byref(plan), batch), lib.fd_plan_min_splits(byref(plan), batch))
+        if min(planned) < 0:
+            check(min(planned))
+        _PLAN_CACHE[key] = planned
+    return planned
+
+
+def item_order_buffer(batch, num_splits, device):
+    """Storage for the work-item order of ``fd_schedule_items`` / ``rope_kv_append(item_order_out=)``."""
+    return torch.empty(2 * batch * num_splits, dtype=torch.int32, device=device)
 
 
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
-            seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True):
+            seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
+            schedule_items=False, item_order=None):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -138,29 +171,19 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     if (k_scale is None) != (v_scale is None):
         raise RuntimeError("k_scale and v_scale must be given together")
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
-    if kv_split == -1 and output_split is None:
-        # the caller left the split count to the library and cannot see the partials: long sequences may get more
-        # than the reference's 32 splits, as long as a split of a full-length sequence keeps 512 tokens
-        num_splits = auto_split_bound(block_table.shape[1] * page_size)
     lib = load_library()
     hstream = stream_handle(stream, q.device.index)
 
     # Partials.  Internal ones are fp32 [B,Hq,S,Dv] + LSE [B,Hq,S] addressed by raw pointers (no tensor views
     # on the hot path); a caller-supplied buffer keeps the reference layout [B,Hq,S,Dv+1].
+    split_adapt = 0
     if output_split is None:
         if plan_splits:
-            # nobody looks at the partials: let the library merge splits (fewer, longer ones)
-            key = (batch, q_heads, kv_heads, q_head_dim, page_size, num_splits, block_table.shape[1], k_cache.dtype,
-                   k_scale is not None, path)
-            planned = _PLAN_CACHE.get(key)
-            if planned is None:
-                plan = _make_params(q, k_cache, block_table, num_splits, soft_cap, FD_F32, FD_F32, k_scale, v_scale,
-                                    path, waves_per_block)
-                planned = lib.fd_plan_splits(byref(plan), batch)
-                if planned < 0:
-                    check(planned)
-                _PLAN_CACHE[key] = planned
-            num_splits = planned
+            # nobody looks at the partials: the library chooses the split count (with kv_split == -1 long sequences
+            # may get more than the reference's 32).  The grid has num_splits slots per sequence; a sequence uses as
+            # many as its own length asks for.
+            num_splits, split_adapt = plan_decode(q, k_cache, block_table, kv_split, k_scale=k_scale, v_scale=v_scale,
+                                                  path=path, waves_per_block=waves_per_block)
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
         direct = (num_splits == 1 and extra_partials is None and not fuse_combine
@@ -194,9 +217,28 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     if seq_order_lens is not None:
         assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
         assert seq_order_lens.numel() == batch
+    # Work-item order ((sequence, range) items, largest first, empty ranges last): given by the caller (the append
+    # launch computed it) or computed here by one scheduling launch.  Internal partials and planned splits only.
+    want_items = (item_order is not None or schedule_items) and split_adapt > 0 and num_splits > 1 and not fuse_combine
+    if want_items and item_order is None and batch > MAX_ITEM_BATCH:
+        want_items = False
+    if schedule_items and not want_items and seq_order is None and num_splits > 1:
+        seq_order = schedule_sequences(kv_lens, stream=stream)   # per-sequence order where items do not apply
     # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
-                     v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0)
+                     v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
+                     split_adapt)
+    if want_items:
+        if item_order is None:
+            item_order = item_order_buffer(batch, num_splits, q.device)
+            if stream is not None:
+                item_order.record_stream(stream)
+            check(lib.fd_schedule_items(hstream, kv_lens.data_ptr(), batch, item_order.data_ptr(), byref(p)))
+        assert item_order.dtype == torch.int32 and item_order.is_contiguous()
+        assert item_order.numel() >= 2 * batch * num_splits
+        p.seq_order_items = 1
+        p.seq_order_lens = None
+        seq_order = item_order
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:
@@ -264,8 +306,8 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
     behind a spinning grid barrier on a fixed 132-workgroup grid; here the device-side
     scheduler orders the sequences longest first and the hardware dispatcher balances the
     workgroups over the CUs, so no co-residency assumption is needed."""
-    if kw.get("seq_order") is None:
-        kw["seq_order"] = schedule_sequences(kv_lens, stream=kw.get("stream"))
+    if kw.get("seq_order") is None and kw.get("item_order") is None:
+        kw["schedule_items"] = True
     return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
                    with_lse_column=False, **kw)
 

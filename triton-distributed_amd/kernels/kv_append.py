@@ -20,7 +20,8 @@ from typing import Optional, Tuple, Union
 import torch
 
 from .._lib import FdParams, FdQkPrep, check, fd_dtype_of, load_library, stream_handle
-from .flash_decode import _decode, _require_cuda
+from .flash_decode import (MAX_FUSED_ITEM_BATCH, SPLIT_ALIGN, _decode, _require_cuda, item_order_buffer,
+                           plan_decode)
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -47,7 +48,8 @@ def _prep_struct(cos_sin, position_ids, head_dim, bsz, seq) -> FdQkPrep:
 def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                    v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                    kv_lens: Optional[torch.Tensor], *, kv_lens_out: Optional[torch.Tensor] = None,
-                   seq_order_out: Optional[torch.Tensor] = None,
+                   seq_order_out: Optional[torch.Tensor] = None, item_order_out: Optional[torch.Tensor] = None,
+                   item_plan: Optional[Tuple[int, int, int]] = None,
                    k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
                    cos_sin: Optional[torch.Tensor] = None, position_ids: Optional[torch.Tensor] = None,
                    q: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None,
@@ -63,15 +65,18 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
     (int32 ``[B]``, not ``kv_lens``) receives the grown lengths; ``seq_order_out`` (int32 ``[2, B]``,
     ``B <= 4096``) the longest-first issue order for the decode that follows (row 0: what ``schedule_sequences``
     would compute, without a launch of its own) and the grown lengths in that order (row 1: the decode's
-    ``seq_order_lens``).  Returns ``q_out`` (or ``None`` without ``q``).
+    ``seq_order_lens``).  ``item_order_out`` (``item_order_buffer(B, num_splits, device)``, ``B <= 256``) with
+    ``item_plan = (num_splits, split_align, split_adapt)`` instead receives the work-item order of the decode that
+    follows (what ``fd_schedule_items`` would compute for the grown lengths; pass it on as ``item_order=``).
+    Returns ``q_out`` (or ``None`` without ``q``).
     """
     lib = load_library()
     append = k_new is not None
     src = k_new if append else q
     if src is None:
         raise RuntimeError("rope_kv_append: neither k_new nor q given")
-    _require_cuda(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out, seq_order_out, cos_sin,
-                  position_ids, q, q_out)
+    _require_cuda(k_new, v_new, k_cache, v_cache, block_table, kv_lens, kv_lens_out, seq_order_out, item_order_out,
+                  cos_sin, position_ids, q, q_out)
     bsz, seq, _, head_dim = src.shape
     p = FdParams()
     p.head_dim = head_dim
@@ -94,8 +99,15 @@ def rope_kv_append(k_new: Optional[torch.Tensor], v_new: Optional[torch.Tensor],
         if kv_lens_out is not None:
             assert kv_lens_out.dtype == torch.int32 and kv_lens_out.is_contiguous() and kv_lens_out.numel() == bsz
         if seq_order_out is not None:
+            assert item_order_out is None
             assert seq_order_out.dtype == torch.int32 and seq_order_out.is_contiguous()
             assert seq_order_out.numel() == 2 * bsz
+        if item_order_out is not None:
+            num_splits, split_align, split_adapt = item_plan
+            assert item_order_out.dtype == torch.int32 and item_order_out.is_contiguous()
+            assert item_order_out.numel() >= 2 * bsz * num_splits
+            p.num_splits, p.split_align, p.split_adapt, p.seq_order_items = num_splits, split_align, split_adapt, 1
+            seq_order_out = item_order_out
         p.page_size = page_size
         p.num_pages = k_cache.shape[0]
         p.max_pages_per_seq = block_table.shape[1]
@@ -215,14 +227,25 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
         assert v is not None
         if kv_lens_out is None:
             kv_lens_out = torch.empty_like(cache_seqlens)
-        order = None
-        if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw:
-            # the append launch also ranks the sequences (longest first) for the decode's issue order
-            order = torch.empty((2, bsz), dtype=torch.int32, device=dev)
-            decode_kw["seq_order"], decode_kw["seq_order_lens"] = order[0], order[1]
+        order = items = item_plan = None
+        if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw \
+                and "item_order" not in decode_kw:
+            # the append launch also computes the decode's issue order: (sequence, range) items, largest first, when
+            # the decode cuts sequences by their own lengths and the batch fits one workgroup; else sequences, longest
+            # first
+            S, adapt = plan_decode(q[:, 0], k_cache, block_table, num_splits if num_splits > 0 else -1,
+                                   k_scale=k_scale, v_scale=v_scale, path=decode_kw.get("path", "auto"),
+                                   waves_per_block=decode_kw.get("waves_per_block", 0))
+            if S > 1 and adapt > 0 and bsz <= MAX_FUSED_ITEM_BATCH and not decode_kw.get("fuse_combine"):
+                items, item_plan = item_order_buffer(bsz, S, dev), (S, SPLIT_ALIGN, adapt)
+                decode_kw["item_order"] = items
+            else:
+                order = torch.empty((2, bsz), dtype=torch.int32, device=dev)
+                decode_kw["seq_order"], decode_kw["seq_order_lens"] = order[0], order[1]
         prep_q = cos_sin_cache is not None or q_norm is not None
         q_rot = rope_kv_append(k, v, k_cache, v_cache, block_table, cache_seqlens, kv_lens_out=kv_lens_out,
-                               seq_order_out=order, k_scale=k_scale, v_scale=v_scale,
+                               seq_order_out=order, item_order_out=items, item_plan=item_plan,
+                               k_scale=k_scale, v_scale=v_scale,
                                cos_sin=cos_sin_cache, position_ids=position_ids, q=q if prep_q else None,
                                q_norm=q_norm, k_norm=k_norm, stream=stream)
         if q_rot is None:
