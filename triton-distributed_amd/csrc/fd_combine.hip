@@ -221,18 +221,31 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_small_kernel(const
   }
 }
 
-// order[rank] = sequence index, sequences ranked by kv_len descending, ties by index.
+// order[rank] = sequence index, sequences ranked by kv_len descending, ties by index.  Every thread ranks its
+// sequence against all others; the lengths go through LDS in chunks so that the inner loop reads four of them per
+// instruction instead of waiting for one scalar load per comparison (1024 sequences: 51 us that way).
+constexpr int kRankChunk = 2048;
+
 __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restrict__ kv_lens, int batch,
                                                           int32_t* __restrict__ order) {
+  __shared__ __align__(16) int32_t s_len[kRankChunk];
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= batch) return;
-  const int mine = kv_lens[i];
+  const int mine = i < batch ? kv_lens[i] : 0;
   int rank = 0;
-  for (int j = 0; j < batch; ++j) {
-    const int other = kv_lens[j];
-    rank += (other > mine) || (other == mine && j < i);
+  for (int j0 = 0; j0 < batch; j0 += kRankChunk) {
+    const int cnt = min(kRankChunk, batch - j0);
+    __syncthreads();
+    for (int j = threadIdx.x; j < kRankChunk; j += blockDim.x) s_len[j] = j < cnt ? kv_lens[j0 + j] : INT32_MIN;
+    __syncthreads();
+    // padding entries (INT32_MIN at indices >= batch) never rank before a real sequence
+#pragma unroll 8
+    for (int j = 0; j < ((cnt + 3) & ~3); j += 4) {
+      const i32x4 other = *(const i32x4*)&s_len[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rank += (other[e] > mine) || (other[e] == mine && j0 + j + e < i);
+    }
   }
-  order[rank] = i;
+  if (i < batch) order[rank] = i;
 }
 
 // One workgroup: the (sequence, range) issue order of a decode step (fd_schedule_items_block).
@@ -245,7 +258,7 @@ __global__ void __launch_bounds__(kMaxItemBatch) fd_schedule_items_kernel(const 
     const int64_t len = kv_lens[j];
     return (int)(len < 0 ? 0 : (len > capacity ? capacity : len));   // as the split kernels clamp it
   };
-  fd_schedule_items_block(threadIdx.x, blockDim.x, batch, len_of, ranges, items, s_key, s_n);
+  fd_schedule_items_block(threadIdx.x, batch, len_of, ranges, items, s_key, s_n);
 }
 
 }  // namespace
@@ -285,7 +298,8 @@ int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, in
 int fd_launch_schedule_items(hipStream_t stream, const int32_t* kv_lens, int batch, int64_t capacity,
                              const RangePlan& ranges, int32_t* items) {
   if (batch > kMaxItemBatch) return FD_ERR_TOO_LARGE;
-  const unsigned threads = (unsigned)((batch + 63) / 64 * 64);
+  unsigned threads = 256;   // the batch rounded up to a power of two; at least 256 to write the list
+  while ((int)threads < batch) threads <<= 1;
   hipLaunchKernelGGL(fd_schedule_items_kernel, dim3(1), dim3(threads), 0, stream, kv_lens, batch, capacity, ranges, items);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }

@@ -13,6 +13,7 @@
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -499,48 +500,91 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
 // Sequences one scheduling workgroup ranks (its LDS holds 12 bytes per sequence).
 constexpr int kMaxItemBatch = 1024;
 
-// Work-item order for the split kernels, computed by ONE workgroup of nthreads threads (batch <= kMaxItemBatch).
-// items[k], k < batch * S, = sequence | range << 16: first the non-empty ranges, sequence by sequence in descending
-// (tokens per range, length) order, ties by index -- all ranges of a sequence have the same size, so this is
-// largest-item-first -- then the empty ranges.  items[batch * S + k] = the length of item k's sequence.
-// len_of(j) = length of sequence j as the decode will see it.  s_key / s_n: LDS, batch entries each.
+// Work-item order for the split kernels, computed by ONE workgroup (batch <= kMaxItemBatch, blockDim.x >= batch
+// rounded up to a power of two, at least 64).  items[k], k < batch * S, = sequence | range << 16: first the non-empty
+// ranges, sequence by sequence in descending order of length, ties by index -- the tokens per range never decrease
+// with the length and all ranges of a sequence have the same size, so this is largest-item-first -- then the empty
+// ranges.  items[batch * S + k] = the length of item k's sequence.  len_of(j) = length of sequence j as the decode
+// will see it.  Up to 64 sequences are ranked by one wave with shuffles (every lane against every other); larger
+// batches by a bitonic sort and a prefix sum in LDS, O(log^2 batch) steps (all pairs took 58 us for 1024 sequences,
+// one workgroup being one CU).  The list is written with consecutive threads on consecutive entries.
+// s_key / s_n: LDS, blockDim.x entries each.
 template <typename LenFn>
-__device__ __forceinline__ void fd_schedule_items_block(int tid, int nthreads, int batch, LenFn len_of,
-                                                        const RangePlan& rp, int32_t* items, uint64_t* s_key,
-                                                        int32_t* s_n) {
-  for (int j = tid; j < batch; j += nthreads) {
-    const int len = len_of(j);
+__device__ __forceinline__ void fd_schedule_items_block(int tid, int batch, LenFn len_of, const RangePlan& rp,
+                                                        int32_t* items, uint64_t* s_key, int32_t* s_n) {
+  int np2 = 64;
+  while (np2 < batch) np2 <<= 1;
+  // n = non-empty ranges of a sequence of len tokens = ceil(len / per) <= S, without an integer division
+  auto ranges_of = [&](int len) {
+    if (len <= 0) return 0;
     const int per = tokens_per_range(len, rp.S, rp.s_magic, rp.s_shift, rp.per_mask, rp.adapt);
-    int n = 0;
-    if (len > 0) {   // n = ceil(len / per) <= S without an integer division
-      n = (int)((float)len / (float)per);
-      while ((int64_t)n * per < len) ++n;
-      while (n > 0 && (int64_t)(n - 1) * per >= len) --n;
+    int n = (int)((float)len / (float)per);
+    while ((int64_t)n * per < len) ++n;
+    while (n > 0 && (int64_t)(n - 1) * per >= len) --n;
+    return n;
+  };
+  // key = length in the high word, ~index in the low word: descending keys = longest first, ties by index;
+  // padding entries (0) sort behind every real one
+  const uint64_t key = tid < batch ? ((uint64_t)(uint32_t)len_of(tid) << 32) | (0xffffffffu - (uint32_t)tid) : 0;
+  if (np2 == 64) {
+    if (tid < 64) {
+      const int n = key ? ranges_of((int)(key >> 32)) : 0;
+      int rank = 0, first = 0;
+      for (int j = 0; j < 64; ++j) {
+        const uint64_t other = ((uint64_t)(uint32_t)__shfl((int)(key >> 32), j) << 32) | (uint32_t)__shfl((int)(uint32_t)key, j);
+        const int n_j = __shfl(n, j);
+        const bool before = other > key;   // keys are distinct
+        rank += before ? 1 : 0;
+        first += before ? n_j : 0;
+      }
+      if (key) {
+        s_key[rank] = key;        // rank = position in the sorted order
+        s_n[rank] = first + n;    // inclusive prefix sum of the non-empty ranges
+      }
     }
-    s_key[j] = ((uint64_t)(uint32_t)per << 32) | (uint32_t)len;
-    s_n[j] = n;
+    __syncthreads();
+  } else {
+    if (tid < np2) s_key[tid] = key;
+    __syncthreads();
+    for (int k = 2; k <= np2; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const int partner = tid ^ j;
+        if (tid < np2 && partner > tid) {
+          const uint64_t x = s_key[tid], y = s_key[partner];
+          const bool descending = (tid & k) == 0;
+          if (descending ? x < y : x > y) {
+            s_key[tid] = y;
+            s_key[partner] = x;
+          }
+        }
+        __syncthreads();
+      }
+    }
+    if (tid < np2) {
+      const uint64_t mine = s_key[tid];
+      s_n[tid] = mine ? ranges_of((int)(mine >> 32)) : 0;
+    }
+    __syncthreads();
+    for (int off = 1; off < np2; off <<= 1) {   // inclusive prefix sum over the ranks
+      const int add = tid < np2 && tid >= off ? s_n[tid - off] : 0;
+      __syncthreads();
+      if (tid < np2) s_n[tid] += add;
+      __syncthreads();
+    }
   }
-  __syncthreads();
   const int total = batch * rp.S;
-  for (int i = tid; i < batch; i += nthreads) {
-    const uint64_t mine = s_key[i];
-    int rank = 0, off = 0, active = 0;
-    for (int j = 0; j < batch; ++j) {
-      const uint64_t other = s_key[j];
-      const int n = s_n[j];
-      const bool before = other > mine || (other == mine && j < i);
-      rank += before ? 1 : 0;
-      off += before ? n : 0;
-      active += n;
-    }
-    const int n_i = s_n[i];
-    const int len_i = (int)(uint32_t)mine;
-    const int empty0 = active + rank * rp.S - off;   // the empty ranges of the sequences before this one
-    for (int t = 0; t < rp.S; ++t) {
-      const int k = t < n_i ? off + t : empty0 + (t - n_i);
-      items[k] = (int32_t)((uint32_t)i | ((uint32_t)t << 16));
-      items[total + k] = len_i;
-    }
+  const int busy = s_n[batch - 1];   // non-empty ranges of the whole batch
+  for (int e = tid; e < total; e += blockDim.x) {
+    const int r = (int)(((uint64_t)(uint32_t)e * rp.s_magic) >> rp.s_shift);   // rank, e / S
+    const int t = e - r * rp.S;                                                 // range of that sequence
+    const uint64_t mine = s_key[r];
+    const int incl = s_n[r];
+    const int first = r ? s_n[r - 1] : 0;      // non-empty ranges of the sequences before this one
+    const int n = incl - first;
+    // the empty ranges of the sequences before this one come first among the empty ones
+    const int k = t < n ? first + t : busy + (r * rp.S - first) + (t - n);
+    items[k] = (int32_t)((0xffffffffu - (uint32_t)mine) | ((uint32_t)t << 16));
+    items[total + k] = (int)(mine >> 32);
   }
 }
 

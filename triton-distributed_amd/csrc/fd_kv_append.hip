@@ -134,8 +134,8 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
     if (a.items) {   // one workgroup: (sequence, range) items, batch <= 256
       __shared__ uint64_t s_key[256];
       __shared__ int32_t s_n[256];
-      fd_schedule_items_block(threadIdx.x, blockDim.x, a.batch, [&](int b) { return (int)grown(b); }, a.ranges,
-                              a.items, s_key, s_n);
+      fd_schedule_items_block(threadIdx.x, a.batch, [&](int b) { return (int)grown(b); }, a.ranges, a.items, s_key,
+                              s_n);
       return;
     }
     // per-sequence order: grown length descending, ties by index

@@ -222,8 +222,10 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     want_items = (item_order is not None or schedule_items) and split_adapt > 0 and num_splits > 1 and not fuse_combine
     if want_items and item_order is None and batch > MAX_ITEM_BATCH:
         want_items = False
-    if schedule_items and not want_items and seq_order is None and num_splits > 1:
-        seq_order = schedule_sequences(kv_lens, stream=stream)   # per-sequence order where items do not apply
+    if schedule_items and not want_items and seq_order is None and num_splits > 1 and batch <= MAX_ITEM_BATCH:
+        # per-sequence order where items do not apply; larger batches are left to the dispatcher (ranking every
+        # sequence against every other one costs more than it gains there)
+        seq_order = schedule_sequences(kv_lens, stream=stream)
     # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
                      v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
