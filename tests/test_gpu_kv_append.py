@@ -339,6 +339,51 @@ def test_append_also_ranks_sequences(fd):
     assert_out_close(out[:, 0], ref)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_serving_loop_ragged_batch_wide_block_table(fd, fp8):
+    """Several decode steps of a ragged batch of 40 sequences through the drop-in call: each step appends one token
+    per sequence, lets the append launch order the decode's (sequence, range) items, and decodes -- in a block table
+    sized for 8192 tokens whose unused entries are garbage.  Oracle on the CPU after every step."""
+    gen = torch.Generator().manual_seed(77)
+    B, Hq, Hkv, D, P, cap_pages = 40, 16, 4, 128, 16, 512
+    lens = torch.randint(0, 1500, (B,), generator=gen, dtype=torch.int32)
+    lens[0], lens[1], lens[2] = 0, 15, 4095
+    need = [-(-(int(n) + 4) // P) for n in lens]
+    pool = sum(need) + 1
+    perm = torch.randperm(pool, generator=gen).to(torch.int32)
+    bt = torch.randint(-3, 1 << 20, (B, cap_pages), generator=gen, dtype=torch.int32)
+    o = 0
+    for b, u in enumerate(need):
+        bt[b, :u] = perm[o:o + u]
+        o += u
+    kc = torch.randn(pool, P, Hkv, D, generator=gen).to(torch.bfloat16)
+    vc = torch.randn(pool, P, Hkv, D, generator=gen).to(torch.bfloat16)
+    k_scale = v_scale = None
+    ref_k, ref_v = kc.clone(), vc.clone()
+    if fp8:
+        k_scale, v_scale = torch.full((Hkv,), 0.02), torch.full((Hkv,), 0.015)
+        ref_k, ref_v = oracle.ref_quantize_fp8(kc.float(), k_scale), oracle.ref_quantize_fp8(vc.float(), v_scale)
+    kc_g, vc_g = ref_k.to(DEV), ref_v.to(DEV)
+    kw = dict(k_scale=k_scale.to(DEV), v_scale=v_scale.to(DEV)) if fp8 else {}
+    lens_g, bt_g = lens.to(DEV), bt.to(DEV)
+    for step in range(4):
+        q = torch.randn(B, 1, Hq, D, generator=gen).to(torch.bfloat16)
+        k = torch.randn(B, 1, Hkv, D, generator=gen).to(torch.bfloat16)
+        v = torch.randn(B, 1, Hkv, D, generator=gen).to(torch.bfloat16)
+        new_lens = oracle.ref_kv_append(k, v, ref_k, ref_v, bt, lens, k_scale=k_scale, v_scale=v_scale)
+        kf = oracle.dequant_fp8_cache(ref_k, k_scale) if fp8 else ref_k.float()
+        vf = oracle.dequant_fp8_cache(ref_v, v_scale) if fp8 else ref_v.float()
+        ref, _ = oracle.ref_paged_attn_lse(q[:, 0].float(), kf, vf, new_lens.tolist(), bt, D ** -0.5)
+        grown = torch.empty_like(lens_g)
+        out = fd.flash_attn_with_kvcache(q.to(DEV), kc_g, vc_g, k=k.to(DEV), v=v.to(DEV), cache_seqlens=lens_g,
+                                         block_table=bt_g, causal=True, kv_lens_out=grown, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(grown.cpu(), new_lens), step
+        assert_out_close(out[:, 0], ref)
+        lens, lens_g = new_lens, grown
+    assert torch.equal(kc_g.cpu().view(torch.uint8), ref_k.view(torch.uint8))
+
+
 def _assert_within_ulps(got, ref, mant_bits, ulps, what):
     got, ref = got.double(), ref.double()
     tol = ref.abs() * (2.0 ** -mant_bits) * ulps + 1e-30

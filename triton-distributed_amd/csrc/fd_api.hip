@@ -367,7 +367,8 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
   // Ranges that follow each sequence's own length leave most slots of a long split list empty: beyond what the
   // small combine kernel takes in one gulp, the empty ranges' workgroups write nothing and the combine derives
   // from kv_lens which slots hold a partial (one more dependent load there, no traffic for the empty ones).
-  const bool skip_empty = p && p->split_adapt > 0 && p->num_splits > kCombineSmallMax && !tickets;
+  const bool skip_empty = p && p->split_adapt > 0 && p->split_adapt < p->num_splits &&
+                          p->num_splits > kCombineSmallMax && !tickets;
   int rc = split_impl("fd_decode", stream, q, k_cache, v_cache, out_split, lse_split, sm_scale, block_table, kv_lens,
                       batch, stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, stride_o_bs,
                       stride_o_h, stride_o_split, stride_table_bs, seq_order, p, &tail, &fused, false, skip_empty);
