@@ -103,11 +103,12 @@ typedef struct fd_params {
                                the reference's.  fd_combine applies the same rule.          */
   int32_t split_adapt;      /* 0: every sequence is cut into num_splits ranges (the reference).
                                k > 0 (a power of two; needs split_align > 0): a range of a sequence
-                               of n tokens holds max(ceil(n / num_splits), min(ceil(n / k), 1024))
-                               tokens -- k ranges up to k * 1024 tokens, 1024-token ranges up to
-                               num_splits * 1024, num_splits ranges beyond -- so a block table
-                               sized for the longest context does not cut a short sequence into
-                               slivers.  The other ranges of the sequence are empty; with more
+                               of n tokens holds max(ceil(n / num_splits), min(ceil(n / k), w))
+                               tokens, w = ceil(n / 8) kept within [1024, 4096] -- at least k
+                               ranges; beyond that 1024-token ranges up to 8 of them, 8 ranges up
+                               to 4096 tokens each, 4096-token ranges up to num_splits of them --
+                               so the ranges of a sequence depend on its own length and not on a
+                               block table sized for the longest context.  The other ranges of the sequence are empty; with more
                                than 16 splits fd_decode does not even write their partials.
                                fd_plan_min_splits gives k.  fd_combine applies the same rule. */
   int32_t seq_order_items;  /* 0: seq_order / seq_order_out is a per-sequence order ([batch], see

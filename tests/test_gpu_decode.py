@@ -585,7 +585,7 @@ def test_item_schedule_matches_oracle_and_is_a_permutation(fd, capacity, kind, b
     assert it[1].tolist() == [lens[b] for b in seq]
 
     def per(n):   # the library's range rule (include/flash_decode.h, fd_params.split_adapt)
-        v = max(-(-n // S), min(-(-n // adapt), 1024))
+        v = max(-(-n // S), min(-(-n // adapt), min(max(-(-n // 8), 1024), 4096)))
         return -(-v // fk.SPLIT_ALIGN) * fk.SPLIT_ALIGN
     busy = [per(lens[b]) * s < lens[b] for b, s in zip(seq, rng_)]
     n_busy = sum(busy)

@@ -227,10 +227,11 @@ constexpr int kMinTokensPerRange = 1024;
 constexpr int kMaxTokensPerRange = 4096;
 
 // Tokens per split range of a sequence of kv_len tokens.  Reference rule: ceil(kv_len / S) (flash_decode.py:193-195).
-// With adapt > 0 (a power of two, the ranges every sequence needs so that the batch fills the chip) a short
-// sequence is not cut into S slivers: per = max(ceil(kv_len / S), min(ceil(kv_len / adapt), 1024)), i.e. adapt
-// ranges up to adapt * 1024 tokens, 1024-token ranges up to S * 1024 tokens, S ranges beyond.  per_mask rounds the
-// result up to the split alignment.  The split kernels and the combine kernel both call this, so they agree on
+// With adapt > 0 (a power of two, the ranges every sequence needs so that the batch fills the chip) the ranges of a
+// sequence follow its own length, not the table's capacity: per = max(ceil(kv_len / S), min(ceil(kv_len / adapt),
+// want)) with want = ceil(kv_len / 8) kept within [1024, 4096] -- at least adapt ranges; beyond that 1024-token
+// ranges up to 8 of them, 8 ranges up to 4096 tokens each, 4096-token ranges up to S of them, S ranges beyond.
+// per_mask rounds the result up to the split alignment.  The split kernels and the combine kernel both call this, so they agree on
 // which ranges are empty.
 __device__ __forceinline__ int tokens_per_range(int kv_len, int S, uint32_t s_magic, uint32_t s_shift, int per_mask,
                                                 int adapt) {
@@ -238,7 +239,8 @@ __device__ __forceinline__ int tokens_per_range(int kv_len, int S, uint32_t s_ma
   int per = (int)(((uint64_t)(uint32_t)(kv_len + S - 1) * s_magic) >> s_shift);
   if (adapt > 0) {
     const int floor_ranges = (kv_len + adapt - 1) >> (31 - __clz(adapt));   // ceil(kv_len / adapt)
-    per = max(per, min(floor_ranges, kMinTokensPerRange));
+    const int want = min(max((kv_len + 7) >> 3, kMinTokensPerRange), kMaxTokensPerRange);
+    per = max(per, min(floor_ranges, want));
   }
   return (per + per_mask) & ~per_mask;
 }
