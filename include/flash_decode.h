@@ -249,7 +249,7 @@ FD_API int fd_schedule_items(void* stream, const int32_t* kv_lens, int32_t batch
  * the workgroup at its full width (sibling KV heads that share 512 bytes of a token row, or head
  * blocks of one KV head), raised (2) until the workgroups are a whole number per CU or at
  * least four per CU, as long as a split of a full-length sequence keeps 512 tokens, and (3) in
- * a batch until no split of a full-length sequence exceeds 4096 tokens (VALU kernel: about
+ * a batch until no split of a full-length sequence exceeds 4096 tokens or 32 splits are reached (VALU kernel: about
  * 2048 waves with four per split instead of (1) and (2)); or a negative fd_status.
  * A caller that passes its own out_split to fd_decode / fd_split_kv keeps exactly
  * params->num_splits splits with the reference's ranges.

@@ -224,6 +224,8 @@ def test_split_plan_policy(fd):
     assert plan(8, 32, 8, 32, 8192) == 32                                      # ... while the grid covers the capacity
     assert fill(64, 32, 8, 32, 8192) == 1 and plan(64, 32, 8, 32, 8192) == 32  # a batch fills the chip by itself
     assert fill(1, 8, 1, 256, 65536) == 256
+    assert plan(64, 32, 8, 256, 65536) == 32       # a table for 1 M tokens: not more than 32 slots per sequence for balance
+    assert plan(2, 32, 8, 256, 65536) == 32 and plan(1, 32, 8, 256, 65536) == 64
     assert fill(0, 32, 8, 32, 512) < 0 and lib.fd_plan_min_splits(None, 1) < 0
     for args in [(3, 16, 16, 32, 83), (7, 6, 1, 5, 1000), (2, 64, 8, 64, 100000)]:
         got = plan(*args)

@@ -79,6 +79,7 @@ constexpr int64_t kTargetWaves = 1024;
 constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
+constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
 
 // Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
 // split) where the caller leaves the choice to the library) and FD_HEADS_PER_BLOCK (members per workgroup).
@@ -428,8 +429,11 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   // (3) in a batch, enough splits that no split of a full-length sequence is longer than kMaxTokensPerSplit: the
   // dispatcher evens out ragged lengths with them
   const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
+  // -- up to kMaxBalanceSplits: the grid has that many slots for EVERY sequence of the batch, and the ones a shorter
+  // sequence leaves empty still cost an issue slot each (a table sized for 1 M tokens would put 256 x batch x KV heads
+  // mostly empty workgroups in front of the chip); sequences beyond 32 x 4096 tokens get longer ranges instead.
   if (batch > 1) {
-    while (s * kMaxTokensPerSplit < max_tokens) s <<= 1;
+    while (s * kMaxTokensPerSplit < max_tokens && s < kMaxBalanceSplits) s <<= 1;
   }
   // Powers of two throughout: with sequence lengths that are powers of two (or multiples of large ones) every split
   // then starts on a tile boundary and the waves of a workgroup get equal runs.
