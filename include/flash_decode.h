@@ -111,6 +111,11 @@ typedef struct fd_params {
                                block table sized for the longest context.  The other ranges of the sequence are empty; with more
                                than 16 splits fd_decode does not even write their partials.
                                fd_plan_min_splits gives k.  fd_combine applies the same rule. */
+  int32_t max_kv_len;       /* 0: unknown.  Else an upper bound of kv_lens that the caller happens to
+                               know on the host (serving engines do): fd_plan_splits and the launch
+                               shape use it instead of the block table's capacity, so a table sized
+                               for the longest context costs nothing.  A hint only: longer sequences
+                               are still decoded in full.  No counterpart in the reference.     */
   int32_t seq_order_items;  /* 0: seq_order / seq_order_out is a per-sequence order ([batch], see
                                fd_schedule and fd_kv_append).  1: it is the work-item order of
                                fd_schedule_items, int32 [2 * batch * num_splits].             */

@@ -540,6 +540,14 @@ def test_short_sequences_in_a_block_table_sized_for_long_contexts(fd, capacity, 
         out, lse = run_decode(fd, wl)
         assert_out_close(out, ref, atol=2e-4 if f32 else 2e-2)
         assert_lse_close(lse, ref_lse, rtol=1e-5 if f32 else 1e-3)
+    # a host-side length hint only changes the launch shape: exact, too small (longer sequences are still decoded in
+    # full) or beyond the capacity
+    wl.kv_split = -1
+    for hint in (max(lens), 100, 10 * capacity):
+        for variant in ("plain", "persistent"):
+            out, lse = run_decode(fd, wl, variant=variant, max_kv_len=hint)
+            assert_out_close(out, ref, atol=2e-4 if f32 else 2e-2)
+            assert_lse_close(lse, ref_lse, rtol=1e-5 if f32 else 1e-3)
     # the merged LSE column and extra partials go through the same ranges
     res, _ = run_decode(fd, wl, variant="intra")
     assert_out_close(res[..., :D], ref, atol=2e-4 if f32 else 2e-2)

@@ -53,6 +53,7 @@ class FdParams(Structure):
         ("path", c_int32), ("waves_per_block", c_int32), ("seq_order_lens", c_void_p),
         ("split_align", c_int32),
         ("split_adapt", c_int32),
+        ("max_kv_len", c_int32),
         ("seq_order_items", c_int32),
     ]
 

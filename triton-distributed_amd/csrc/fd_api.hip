@@ -71,6 +71,13 @@ int check_split_adapt(const char* fn, const fd_params* p) {
   return FD_OK;
 }
 
+// Longest sequence the launch shape is planned for: the block table's capacity, or the caller's smaller hint.
+// A sequence that is longer all the same is still decoded in full (its ranges just get longer than planned).
+int64_t planned_tokens(const fd_params* p) {
+  const int64_t cap = (int64_t)p->max_pages_per_seq * p->page_size;
+  return p->max_kv_len > 0 && p->max_kv_len < cap ? p->max_kv_len : cap;
+}
+
 // Launch-shape policy, from sweeps on one MI355X (256 CUs): the MFMA kernels stream best with about
 // 1024 waves in flight (16 KB of loads each), the VALU kernel with about 2048 (8 KB each), each walking
 // a long token range (every wave pays a fixed prologue / epilogue, and every split adds a partial for
@@ -179,7 +186,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
       stride_v_tok * kvsz >= ((int64_t)1 << 31))
     return fail(FD_ERR_INVALID_ARG, "%s: token stride out of range", fn);
   const int G = p->q_heads / p->kv_heads;
-  int64_t max_tok_split = ((int64_t)p->max_pages_per_seq * p->page_size + p->num_splits - 1) / p->num_splits;
+  int64_t max_tok_split = (planned_tokens(p) + p->num_splits - 1) / p->num_splits;
   if (p->split_adapt > 0 && max_tok_split < kMinTokensPerRange)   // ranges by each sequence's own length
     max_tok_split = kMinTokensPerRange;
 
@@ -391,7 +398,7 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
   const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
-  const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
+  const int64_t max_tokens = planned_tokens(p);
   int64_t s = 1;
   if (mfma) {
     // (1) one workgroup per CU at the full member width (sibling KV heads, or head blocks of one KV head): measured
@@ -428,7 +435,7 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   if (s < 0) return (int)s;
   // (3) in a batch, enough splits that no split of a full-length sequence is longer than kMaxTokensPerSplit: the
   // dispatcher evens out ragged lengths with them
-  const int64_t max_tokens = (int64_t)p->max_pages_per_seq * p->page_size;
+  const int64_t max_tokens = planned_tokens(p);
   // -- up to kMaxBalanceSplits: the grid has that many slots for EVERY sequence of the batch, and the ones a shorter
   // sequence leaves empty still cost an issue slot each (a table sized for 1 M tokens would put 256 x batch x KV heads
   // mostly empty workgroups in front of the chip); sequences beyond 32 x 4096 tokens get longer ranges instead.

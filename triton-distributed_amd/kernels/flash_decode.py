@@ -98,7 +98,8 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 
 
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
-                 waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0) -> FdParams:
+                 waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0,
+                 max_kv_len=0) -> FdParams:
     p = FdParams()
     p.q_heads = q.shape[1]
     p.kv_heads = k_cache.shape[2]
@@ -120,6 +121,7 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
     p.split_align = split_align
     p.split_adapt = split_adapt
     p.seq_order_items = seq_order_items
+    p.max_kv_len = max_kv_len
     return p
 
 
@@ -127,20 +129,32 @@ MAX_ITEM_BATCH = 1024       # sequences fd_schedule_items ranks in one launch
 MAX_FUSED_ITEM_BATCH = 256  # ... and fd_kv_append in its trailing workgroup
 
 
-def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=None, path="auto", waves_per_block=0):
+def _hint(max_kv_len, capacity):
+    """The host-side length hint as the library takes it: 0 = none, else rounded up to a multiple of 1024 tokens so
+    that a growing batch does not re-plan at every step."""
+    if not max_kv_len or max_kv_len >= capacity:
+        return 0
+    return min(capacity, -(-int(max_kv_len) // 1024) * 1024)
+
+
+def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=None, path="auto", waves_per_block=0,
+                max_kv_len=None):
     """The split plan of a decode step whose partials stay inside the library: ``(num_splits, split_adapt)`` --
     grid slots per sequence and the ranges every sequence gets however short it is (``fd_plan_splits``,
-    ``fd_plan_min_splits``; cached by shape).  ``kv_split`` is the caller's bound, -1 leaves it to the library."""
+    ``fd_plan_min_splits``; cached by shape).  ``kv_split`` is the caller's bound, -1 leaves it to the library;
+    ``max_kv_len`` an upper bound of the lengths known on the host (else the block table's capacity counts)."""
     batch, q_heads, q_head_dim = q.shape
     page_size, kv_heads = k_cache.shape[1], k_cache.shape[2]
-    bound = auto_split_bound(block_table.shape[1] * page_size) if kv_split == -1 else kv_split
+    capacity = block_table.shape[1] * page_size
+    hint = _hint(max_kv_len, capacity)
+    bound = auto_split_bound(hint or capacity) if kv_split == -1 else kv_split
     key = (batch, q_heads, kv_heads, q_head_dim, page_size, bound, block_table.shape[1], k_cache.dtype,
-           k_scale is not None, path)
+           k_scale is not None, path, hint)
     planned = _PLAN_CACHE.get(key)
     if planned is None:
         lib = load_library()
         plan = _make_params(q, k_cache, block_table, bound, 0.0, FD_F32, FD_F32, k_scale, v_scale, path,
-                            waves_per_block)
+                            waves_per_block, max_kv_len=hint)
         planned = (lib.fd_plan_splits(byref(plan), batch), lib.fd_plan_min_splits(byref(plan), batch))
         if min(planned) < 0:
             check(min(planned))
@@ -156,7 +170,7 @@ def item_order_buffer(batch, num_splits, device):
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
             seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
-            schedule_items=False, item_order=None):
+            schedule_items=False, item_order=None, max_kv_len=None):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -183,7 +197,7 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             # may get more than the reference's 32).  The grid has num_splits slots per sequence; a sequence uses as
             # many as its own length asks for.
             num_splits, split_adapt = plan_decode(q, k_cache, block_table, kv_split, k_scale=k_scale, v_scale=v_scale,
-                                                  path=path, waves_per_block=waves_per_block)
+                                                  path=path, waves_per_block=waves_per_block, max_kv_len=max_kv_len)
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
         direct = (num_splits == 1 and extra_partials is None and not fuse_combine
@@ -229,7 +243,7 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
                      v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
-                     split_adapt)
+                     split_adapt, 0, _hint(max_kv_len, block_table.shape[1] * page_size))
     if want_items:
         if item_order is None:
             item_order = item_order_buffer(batch, num_splits, q.device)
@@ -288,7 +302,9 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
 
     ``q_lens`` is accepted and ignored, as in the reference; so is ``workspace``, unless it is a
     contiguous float32 GPU tensor of at least ``B*Hq*S*(Dv+1)`` elements, in which case the split
-    partials live in it instead of in freshly allocated memory.
+    partials live in it instead of in freshly allocated memory.  Keyword ``max_kv_len=``: an upper bound of
+    ``kv_lens`` that the caller knows on the host; the launch shape is then planned for it instead of for the block
+    table's capacity (a hint only: longer sequences are still decoded in full).
     """
     return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
                    with_lse_column=False, **kw)

@@ -235,7 +235,8 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
             # first
             S, adapt = plan_decode(q[:, 0], k_cache, block_table, num_splits if num_splits > 0 else -1,
                                    k_scale=k_scale, v_scale=v_scale, path=decode_kw.get("path", "auto"),
-                                   waves_per_block=decode_kw.get("waves_per_block", 0))
+                                   waves_per_block=decode_kw.get("waves_per_block", 0),
+                                   max_kv_len=decode_kw.get("max_kv_len"))
             if S > 1 and adapt > 0 and bsz <= MAX_FUSED_ITEM_BATCH and not decode_kw.get("fuse_combine"):
                 items, item_plan = item_order_buffer(bsz, S, dev), (S, SPLIT_ALIGN, adapt)
                 decode_kw["item_order"] = items
