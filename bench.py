@@ -34,7 +34,8 @@ def parse_args():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (2 = Llama-3-8B shape, the one the metric is quoted on)")
     ap.add_argument("--pools", type=int, default=4, help="independent KV pools the steps rotate over")
     ap.add_argument("--clock-ramp-ms", type=float, default=250.0,
-                    help="untimed run of the step before the warm-up steps, so that an idle GPU reaches its clocks")
+                    help="least untimed run of the step before the warm-up steps (until its time has settled, at "
+                         "most 20 times as long), so that an idle or just vacated GPU is in its steady state")
     ap.add_argument("--variant", default="plain", choices=["plain", "persistent"])
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--waves", type=int, default=0)
@@ -249,16 +250,28 @@ def main():
         return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
 
     # ---- whole-step timing
-    # An idle GPU takes a while to reach its clocks, longer than a warm-up of a few milliseconds: run the step untimed
-    # for a quarter of a second first (the first measurement on a freshly acquired machine otherwise reads ~4 % low
-    # against the same command a minute later).
+    # An idle GPU takes a while to reach its clocks, and a machine on which a process has just released tens of GiB of
+    # device memory is busy with that for a few seconds more (measured: the first run after such a process read 5 %
+    # slow, the same command seconds later did not).  Run the step untimed, in batches timed with events, until the
+    # batch time has settled (three batches in a row within 1 % of the best one) -- at least --clock-ramp-ms, at most
+    # 20 times that.
     t_ramp = time.perf_counter()
-    i_ramp = 0
-    while time.perf_counter() - t_ramp < args.clock_ramp_ms * 1e-3:
-        for _ in range(50):
+    i_ramp, best, settled = 0, float("inf"), 0
+    r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    while args.clock_ramp_ms > 0:
+        r0.record()
+        for _ in range(100):
             step(i_ramp)
             i_ramp += 1
+        r1.record()
         torch.cuda.synchronize()
+        took = r0.elapsed_time(r1)
+        settled = settled + 1 if 0.99 * best <= took <= 1.01 * best else 0
+        best = min(best, took)
+        waited_ms = (time.perf_counter() - t_ramp) * 1e3
+        if (waited_ms >= args.clock_ramp_ms and settled >= 3) or waited_ms >= 20 * args.clock_ramp_ms:
+            break
+    ramp_ms = (time.perf_counter() - t_ramp) * 1e3
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -372,7 +385,7 @@ def main():
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
-        "clock_ramp_ms": args.clock_ramp_ms,
+        "clock_ramp_ms": round(ramp_ms),
         "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "kernel_us": round(split_us, 3)},

@@ -41,3 +41,35 @@ struct Mma<_Float16> {
   }
 };
 
+// One online-softmax step of the "lane c = head c" layout shared by the MFMA split kernels.  x[0..N) are this lane's
+// scores of head c for N tokens of the tile, in the base-2 domain, masked tokens = -inf; the four wave rows hold
+// different tokens of the same head.  Updates the running max m (identical in the four rows) and the lane's share l
+// of the running sum, replaces x by the probabilities 2^(x - m), and returns the factor the accumulators of head c
+// have to be multiplied by; moved = some lane's max moved (wave-uniform), i.e. whether that rescale is needed at all.
+// Every tile holds at least one valid token, so the new max is finite.
+template <int N>
+__device__ __forceinline__ float fd_softmax_step(float (&x)[N], float& m, float& l, bool& moved) {
+  float t[N];   // pairwise tree: a short dependency chain
+#pragma unroll
+  for (int i = 0; i < N; ++i) t[i] = x[i];
+#pragma unroll
+  for (int stride = 1; stride < N; stride *= 2) {
+#pragma unroll
+    for (int i = 0; i + stride < N; i += 2 * stride) t[i] = fmaxf(t[i], t[i + stride]);
+  }
+  float mx = t[0];
+  mx = fmaxf(mx, __shfl_xor(mx, 16));
+  mx = fmaxf(mx, __shfl_xor(mx, 32));
+  const float m_new = fmaxf(m, mx);
+  const float alpha = fd_exp2(m - m_new);
+  float psum = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    x[i] = fd_exp2(x[i] - m_new);
+    psum += x[i];
+  }
+  l = l * alpha + psum;
+  moved = __any(m_new > m);
+  m = m_new;
+  return alpha;
+}

@@ -194,23 +194,12 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
         const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
         x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
       }
-      float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m[nb], mx);  // finite: every tile holds at least one valid token
-      const float alpha = fd_exp2(m[nb] - m_new);
-      float psum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        x[i] = fd_exp2(x[i] - m_new);
-        psum += x[i];
-      }
-      l[nb] = l[nb] * alpha + psum;
-      if (__any(m_new > m[nb])) {
+      bool moved;
+      const float alpha = fd_softmax_step(x, m[nb], l[nb], moved);
+      if (moved) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[nb][j] *= alpha;
       }
-      m[nb] = m_new;
 #pragma unroll
       for (int e = 0; e < 4; ++e) pop[nb][e] = Mma<T>::pack(x[2 * e], x[2 * e + 1]);
     }

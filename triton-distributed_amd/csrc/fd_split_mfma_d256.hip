@@ -163,25 +163,14 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
       }
       x[i] = (full || n0 + 4 * g + i < w.end) ? v : -INFINITY;
     }
-    float mx = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m, mx);  // finite: every tile holds at least one valid token
-    const float alpha = fd_exp2(m - m_new);
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x[i] = fd_exp2(x[i] - m_new);
-      psum += x[i];
-    }
-    l = l * alpha + psum;
-    if (__any(m_new > m)) {
+    bool moved;
+    const float alpha = fd_softmax_step(x, m, l, moved);
+    if (moved) {
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[h][j] *= alpha;
     }
-    m = m_new;
     u32x2 pop;  // P^T as the B operand: k = 4g + e <-> token 4g + e
     pop[0] = Mma<T>::pack(x[0], x[1]);
     pop[1] = Mma<T>::pack(x[2], x[3]);

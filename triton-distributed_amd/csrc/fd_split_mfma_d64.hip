@@ -150,25 +150,12 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d64_kernel(const SplitArg
         x[4 * tt + i] = (full || n0 + 16 * tt + 4 * g + i < w.end) ? v : -INFINITY;
       }
     }
-    float mx = x[0];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, x[i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = fd_exp2(m - m_new);
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      x[i] = fd_exp2(x[i] - m_new);
-      psum += x[i];
-    }
-    l = l * alpha + psum;
-    if (__any(m_new > m)) {
+    bool moved;
+    const float alpha = fd_softmax_step(x, m, l, moved);
+    if (moved) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[j] *= alpha;
     }
-    m = m_new;
     u32x4 pop[2];  // P^T B operands: block kblk, element e <-> token 16*(2kblk + e/4) + 4g + e%4
 #pragma unroll
     for (int kblk = 0; kblk < 2; ++kblk)
