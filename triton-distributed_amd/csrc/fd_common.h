@@ -331,13 +331,31 @@ __device__ __forceinline__ int page_index(const SplitArgs& a, int n) {
   return (int)(((uint64_t)(uint32_t)n * a.div_magic) >> a.div_shift);
 }
 
+// Block-table entry and in-page slot of the token a lane looks up for tile t of its wave's run (TILE tokens per
+// tile): token start + t * TILE + tok_lane, clamped to the last token of the range (the scores of the clamped
+// tokens are masked).  The table entry is returned raw: its arithmetic is left to the consumer one iteration later,
+// so that the load stays in flight across the tile that is being processed.
+template <int TILE>
+__device__ __forceinline__ int fd_tile_slot(const SplitArgs& a, const WorkItem& w, const int32_t* bt_row, int t,
+                                            int tok_lane, int& slot) {
+  int n = w.start + t * TILE + tok_lane;
+  n = min(n, w.end - 1);
+  const int pidx = page_index(a, n);
+  slot = n - pidx * a.P;
+  return bt_row[pidx];
+}
+
+// Flat cache row page * P + slot of a raw table entry, the page id clamped into the pool so that a corrupt table
+// cannot fault the GPU.
+__device__ __forceinline__ int fd_flat_row(const SplitArgs& a, int page, int slot) {
+  return min(max(page, 0), a.num_pages - 1) * a.P + slot;
+}
+
 // Flat cache row of logical token n of sequence b: page*P + n%P, with the page id
 // clamped into the pool so that a corrupt table entry cannot fault the GPU.
 __device__ __forceinline__ int token_row(const SplitArgs& a, const int32_t* bt_row, int n) {
-  int pidx = page_index(a, n);
-  int page = bt_row[pidx];
-  page = min(max(page, 0), a.num_pages - 1);
-  return page * a.P + (n - pidx * a.P);
+  const int pidx = page_index(a, n);
+  return fd_flat_row(a, bt_row[pidx], n - pidx * a.P);
 }
 
 // Merges the per-wave partial states of a workgroup and stores one normalised partial (out, lse)

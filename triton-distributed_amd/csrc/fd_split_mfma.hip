@@ -93,23 +93,14 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
   float scale2 = a.sm_scale * FD_LOG2E;  // scores are kept in the base-2 domain
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
-  // Block-table entry and in-page slot of tile t for this lane: lane (l & 31) owns token
-  // start + 32t + (l & 31); tokens past the split end are clamped to the last valid token (their
-  // scores are masked).  The table entry is returned raw: its arithmetic is done by the consumer
-  // one iteration later, so the load stays in flight across the tile that is being processed.
-  auto tile_slot = [&](int t, int& slot) -> int {
-    int n = w.start + t * kTile + (lane & 31);
-    n = min(n, w.end - 1);
-    const int pidx = page_index(a, n);
-    slot = n - pidx * a.P;
-    return bt_row[pidx];
-  };
+  // lane (l & 31) looks up token start + 32t + (l & 31)
+  auto tile_slot = [&](int t, int& slot) -> int { return fd_tile_slot<kTile>(a, w, bt_row, t, lane & 31, slot); };
 
   u32x4 kraw[8], vraw[8];
   int rows[8];
   auto fetch_rows = [&](int page, int slot) {
     // flat cache row = page * P + slot, page clamped into the pool so a corrupt table cannot fault
-    const int rv = min(max(page, 0), a.num_pages - 1) * a.P + slot;
+    const int rv = fd_flat_row(a, page, slot);
 #pragma unroll
     for (int i = 0; i < 8; ++i) rows[i] = __shfl(rv, 4 * g + (i & 3) + 16 * (i >> 2));
   };

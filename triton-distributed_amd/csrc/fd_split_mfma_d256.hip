@@ -84,18 +84,12 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
 
   // lane (l & 15) owns token start + 16t + (l & 15) of tile t; the raw table entry is returned and turned
   // into a row by the consumer one iteration later (the load stays in flight across a tile)
-  auto tile_slot = [&](int t, int& slot) -> int {
-    int n = w.start + t * kTile + c;
-    n = min(n, w.end - 1);
-    const int pidx = page_index(a, n);
-    slot = n - pidx * a.P;
-    return bt_row[pidx];
-  };
+  auto tile_slot = [&](int t, int& slot) -> int { return fd_tile_slot<kTile>(a, w, bt_row, t, c, slot); };
 
   u32x4 kraw[8], vraw[8];   // [2 * i + h]: token 4g + i, half h
   int rows[4];
   auto fetch_rows = [&](int page, int slot) {
-    const int rv = min(max(page, 0), a.num_pages - 1) * a.P + slot;
+    const int rv = fd_flat_row(a, page, slot);
 #pragma unroll
     for (int i = 0; i < 4; ++i) rows[i] = __shfl(rv, 4 * g + i);
   };

@@ -70,15 +70,9 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d64_kernel(const SplitArg
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
   // lane l owns token start + 64t + l of tile t (clamped to the last valid token of the split)
-  auto tile_slot = [&](int t, int& slot) -> int {
-    int n = w.start + t * kTile + lane;
-    n = min(n, w.end - 1);
-    const int pidx = page_index(a, n);
-    slot = n - pidx * a.P;
-    return bt_row[pidx];
-  };
+  auto tile_slot = [&](int t, int& slot) -> int { return fd_tile_slot<kTile>(a, w, bt_row, t, lane, slot); };
   auto flat_row = [&](int page, int slot) -> int {
-    return min(max(page, 0), a.num_pages - 1) * a.P + slot;
+    return fd_flat_row(a, page, slot);
   };
 
   u32x4 kraw[8];

@@ -69,18 +69,12 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
   const float scale2 = kq_scale * FD_LOG2E;
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
-  auto tile_slot = [&](int t, int& slot) -> int {
-    int n = w.start + t * kTile + (lane & 31);
-    n = min(n, w.end - 1);
-    const int pidx = page_index(a, n);
-    slot = n - pidx * a.P;
-    return bt_row[pidx];
-  };
+  auto tile_slot = [&](int t, int& slot) -> int { return fd_tile_slot<kTile>(a, w, bt_row, t, lane & 31, slot); };
 
   u32x4 kraw[8], vraw[8];
   int rows[8];
   auto fetch_rows = [&](int page, int slot) {
-    const int rv = min(max(page, 0), a.num_pages - 1) * a.P + slot;
+    const int rv = fd_flat_row(a, page, slot);
 #pragma unroll
     for (int i = 0; i < 8; ++i) rows[i] = __shfl(rv, 4 * g + (i & 3) + 16 * (i >> 2));
   };
