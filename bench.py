@@ -197,6 +197,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the flash-decode library has no CPU path", file=sys.stderr)
         sys.exit(2)
+    importlib.import_module("triton-distributed_amd.build").ensure_built()   # loads what is built; builds only if nothing is
     fd.load_library()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

@@ -25,5 +25,7 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(scope="session")
 def fd():
-    """The package under test (its directory name is not an identifier)."""
+    """The package under test (its directory name is not an identifier).  The library is used as built; only a tree
+    in which nothing has been built yet gets one build."""
+    importlib.import_module("triton-distributed_amd.build").ensure_built()
     return importlib.import_module("triton-distributed_amd")

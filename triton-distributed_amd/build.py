@@ -87,3 +87,14 @@ if __name__ == "__main__":
     ns = ap.parse_args()
     print(build(force=ns.force, verbose=not ns.quiet))
     sys.exit(0)
+
+
+def ensure_built(verbose: bool = False) -> str:
+    """For tests, the smoke check and the bench: the library as it is if it has been built (or FD_LIBRARY_PATH names
+    one), else one build.  The package itself never builds behind the caller's back: ``load_library`` raises."""
+    override = os.environ.get("FD_LIBRARY_PATH")
+    if override:
+        return override
+    if os.path.exists(LIB_PATH):
+        return LIB_PATH
+    return build(force=False, verbose=verbose)
