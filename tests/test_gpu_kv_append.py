@@ -375,8 +375,9 @@ def test_serving_loop_ragged_batch_wide_block_table(fd, fp8):
         vf = oracle.dequant_fp8_cache(ref_v, v_scale) if fp8 else ref_v.float()
         ref, _ = oracle.ref_paged_attn_lse(q[:, 0].float(), kf, vf, new_lens.tolist(), bt, D ** -0.5)
         grown = torch.empty_like(lens_g)
+        hint = dict(max_kv_len=int(new_lens.max())) if step % 2 else {}   # every other step with the host-side hint
         out = fd.flash_attn_with_kvcache(q.to(DEV), kc_g, vc_g, k=k.to(DEV), v=v.to(DEV), cache_seqlens=lens_g,
-                                         block_table=bt_g, causal=True, kv_lens_out=grown, **kw)
+                                         block_table=bt_g, causal=True, kv_lens_out=grown, **hint, **kw)
         torch.cuda.synchronize()
         assert torch.equal(grown.cpu(), new_lens), step
         assert_out_close(out[:, 0], ref)
