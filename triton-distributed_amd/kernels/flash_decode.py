@@ -324,8 +324,8 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
     behind a spinning grid barrier on a fixed 132-workgroup grid; here the device-side
     scheduler orders the sequences longest first and the hardware dispatcher balances the
     workgroups over the CUs, so no co-residency assumption is needed."""
-    if kw.get("seq_order") is None and kw.get("item_order") is None:
-        kw["schedule_items"] = True
+    if kw.get("seq_order") is None and kw.get("item_order") is None and q.shape[0] > 1:
+        kw["schedule_items"] = True   # a single sequence has nothing to order
     return _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine, kv_split,
                    with_lse_column=False, **kw)
 
