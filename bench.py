@@ -375,8 +375,10 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp8-e4m3 KV / bf16 Q, fp32 accumulate" if wl.k_scale is not None else
-                 f"{str(wl.q.dtype).replace('torch.', '')} KV+Q, fp32 accumulate",
+        # the type the path computes in: the MFMA operands' (KV dequantised to it), or f32 on the VALU path
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[wl.q.dtype],
+        "dtype_detail": ("fp8-e4m3 KV dequantised to the query's " if wl.k_scale is not None else "KV and Q ")
+                        + f"{str(wl.q.dtype).replace('torch.', '')}, fp32 accumulate and softmax",
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "q_heads": Hq, "kv_heads": wl.k_cache.shape[2], "head_dim": D,
                    "page_size": wl.k_cache.shape[1], "kv_splits": S, "kv_splits_used": S_eff,
