@@ -56,3 +56,49 @@ def test_random_shape(fd, i):
         lse_rtol = 1e-5 if fp32 else 1e-3
     assert_out_close(out, ref, atol=2e-4 if fp32 else 2e-2)
     assert_lse_close(lse, ref_lse, rtol=lse_rtol)
+
+
+# ---- second sweep: batches up to 80 sequences in block tables wider than the sequences (garbage beyond the used
+# pages), the library's own split count, length hints, the item scheduler, groups up to 40 query heads
+SERVING_CASES = 100
+
+
+def _serving_case(i):
+    rng = random.Random(12000 + i)
+    D = rng.choice([64, 128, 128, 128, 256])
+    kind = rng.choice(["bf16", "fp16", "fp8"]) if D != 64 else rng.choice(["bf16", "fp16"])
+    Hkv = rng.choice([1, 2, 4, 8])
+    G = rng.choice([1, 4, 4, 7, 8, 16, 24, 40]) if D == 128 else rng.choice([1, 4, 8])
+    B = rng.choice([1, 2, 6, 17, 40, 80])
+    P = rng.choice([1, 16, 16, 64])
+    top = rng.choice([40, 700, 3000])
+    lens = [rng.choice([0, 1, 63, 64, 65, 1023, 1024, 1025]) if rng.random() < 0.3 else rng.randint(1, top)
+            for _ in range(B)]
+    lens[0] = max(lens[0], 1)
+    widen = rng.choice([1, 1, 8, 64, 700])
+    hint = rng.choice([None, None, "exact", "low", "high"])
+    return dict(D=D, kind=kind, Hq=Hkv * G, Hkv=Hkv, P=P, lens=lens, widen=widen, hint=hint,
+                kv_split=rng.choice([-1, -1, 32, 4]), variant=rng.choice(["plain", "persistent", "persistent"]),
+                soft_cap=rng.choice([0.0, 0.0, 50.0]))
+
+
+@pytest.mark.parametrize("i", range(SERVING_CASES))
+def test_random_serving_shape(fd, i):
+    c = _serving_case(i)
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp8": torch.bfloat16}[c["kind"]]
+    wl = fd.utils.make_paged_workload(f"serve{i}", c["lens"], c["Hq"], c["Hkv"], c["D"], c["P"], dtype, c["kv_split"],
+                                      seed=15000 + i, soft_cap=c["soft_cap"], fp8_kv=c["kind"] == "fp8")
+    used = wl.block_table.shape[1]
+    gen = torch.Generator().manual_seed(i)
+    wide = torch.randint(-9, 1 << 28, (len(c["lens"]), used * c["widen"]), generator=gen, dtype=torch.int32)
+    for b, n in enumerate(c["lens"]):
+        pages = -(-n // c["P"])
+        wide[b, :pages] = wl.block_table[b, :pages]
+    wl.block_table = wide
+    kw = {}
+    if c["hint"] is not None:
+        kw["max_kv_len"] = {"exact": max(c["lens"]), "low": max(1, max(c["lens"]) // 3), "high": 10 ** 7}[c["hint"]]
+    ref, ref_lse = oracle_decode(wl)
+    out, lse = run_decode(fd, wl, variant=c["variant"], **kw)
+    assert_out_close(out, ref, atol=2e-2)
+    assert_lse_close(lse, ref_lse, rtol=1e-3)
