@@ -83,12 +83,17 @@ def test_other_dtypes_and_groups(fd, dtype, num_heads, block_size):
 
 # ---- groups above 16 query heads: two 16-head blocks per wave (head_dim 128, 16-bit cache), further blocks as
 # sibling waves; the last block may be partly or wholly padding
-@pytest.mark.parametrize("dtype,soft_cap", [(torch.bfloat16, 0), (torch.float16, 30)])
+@pytest.mark.parametrize("dtype,soft_cap,fp8", [(torch.bfloat16, 0, False), (torch.float16, 30, False),
+                                                (torch.bfloat16, 0, True), (torch.float16, 50, True)])
 @pytest.mark.parametrize("num_heads", [(32, 1), (64, 2), (17, 1), (48, 1), (64, 1), (80, 1), (132, 1)])
 @pytest.mark.parametrize("waves,fuse,plan", [(0, False, True), (1, False, False), (2, True, False), (4, False, False),
                                              (8, True, True)])
-def test_two_head_blocks_per_wave(fd, dtype, soft_cap, num_heads, waves, fuse, plan):
-    wl = _grid_workload(fd, [1320, 18, 463, 2049, 33, 0, 1], num_heads, 128, 16, dtype, soft_cap, seed=17)
+def test_two_head_blocks_per_wave(fd, dtype, soft_cap, fp8, num_heads, waves, fuse, plan):
+    if fp8:
+        wl = fd.utils.make_paged_workload("two_blocks_fp8", [1320, 18, 463, 2049, 33, 0, 1], num_heads[0], num_heads[1],
+                                          128, 16, dtype, 32, seed=17, soft_cap=float(soft_cap), fp8_kv=True)
+    else:
+        wl = _grid_workload(fd, [1320, 18, 463, 2049, 33, 0, 1], num_heads, 128, 16, dtype, soft_cap, seed=17)
     out, lse = run_decode(fd, wl, path="mfma", waves_per_block=waves, fuse_combine=fuse, plan_splits=plan)
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)

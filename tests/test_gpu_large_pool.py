@@ -53,6 +53,7 @@ CASES = [  # name, Hq, Hkv, D, P, dtype, fp8, path
     ("mfma_bf16_d128", 32, 8, 128, 16, torch.bfloat16, False, "auto"),
     ("mfma_fp16_d128_two_blocks", 64, 2, 128, 16, torch.float16, False, "auto"),
     ("mfma_fp8_d128", 64, 8, 128, 16, torch.bfloat16, True, "auto"),
+    ("mfma_fp8_d128_two_blocks", 64, 2, 128, 16, torch.float16, True, "auto"),
     ("mfma_bf16_d256", 16, 4, 256, 16, torch.bfloat16, False, "auto"),
     ("mfma_fp8_d256", 16, 4, 256, 16, torch.bfloat16, True, "auto"),
     ("mfma_bf16_d64", 32, 8, 64, 16, torch.bfloat16, False, "auto"),

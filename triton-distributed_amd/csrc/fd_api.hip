@@ -56,8 +56,12 @@ bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
 // Query-head slots of one head block of the MFMA kernels: 16 (one MFMA column block per wave), or 32 where the kernel
 // serves two column blocks per wave from one pass over K and V and the group is large enough to use them.
 int mfma_head_block(int head_dim, int group, int kv_dtype) {
-  const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
-  return (group > 16 && head_dim == 128 && kv16) ? 32 : 16;
+  if (head_dim != 128) return 16;
+  if (kv_dtype == FD_F16 || kv_dtype == FD_BF16) return group > 16 ? 32 : 16;
+  // fp8: two sibling waves of 16 heads each still beat one two-block wave (G = 32: 47.3 vs 52.1 us on config 2's
+  // shape); beyond that two two-block waves beat four sibling waves (G = 64: 62.5 vs 77.0 us)
+  if (kv_dtype == FD_FP8_E4M3) return group > 32 ? 32 : 16;
+  return 16;
 }
 
 // fd_params.split_adapt: 0, or a power of two together with a split alignment and a power-of-two split count.

@@ -30,12 +30,17 @@ namespace {
 constexpr int kD = 128;
 constexpr int kTile = 64;         // tokens per tile
 constexpr int kKRow = 144;        // LDS pitch of a staged fp8 K row in bytes (128 + 16 pad)
-constexpr int kWaveLds = kTile * kKRow;  // 9216 B per wave, reused for the wave's partial result
-constexpr int kHB = 16;
-static_assert(kWaveLds >= (kHB * kD + 2 * kHB) * 4, "partial result must fit in the K staging buffer");
+constexpr int kKTile = kTile * kKRow;   // 9216 B of staged K per wave
+// LDS per wave: the K staging buffer, reused for the wave's partial result (16*NB heads x (128 + 2) floats)
+constexpr int wave_lds(int nb) { return nb == 1 ? kKTile : (16 * nb * kD + 2 * 16 * nb) * 4; }
+static_assert(wave_lds(1) >= (16 * kD + 2 * 16) * 4 && wave_lds(2) >= kKTile, "partial result and K tile share the buffer");
 
-template <typename T, bool SOFTCAP>
-__global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs a) {
+// NB = 2 (groups above 16 query heads): a wave serves two 16-head blocks from the same converted K operands and the
+// same converted, transposed V operands; only the MFMAs and the softmax are done per block.
+template <typename T, bool SOFTCAP, int NB>
+__global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(const SplitArgs a) {
+  constexpr int kHB = 16 * NB;            // head slots per wave
+  constexpr int kWaveLds = wave_lds(NB);
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -51,17 +56,17 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
   const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 
-  const int head_in_group = w.hb * kHB + c;
-  const bool head_ok = head_in_group < a.G;
-  const int head = w.kvh * a.G + head_in_group;
-
-  u32x4 qop[4];  // Q as the MFMA B operand: lane (g, c) holds Q[head c][32*ks + 8g .. +7]
-  {
+  u32x4 qop[NB][4];  // Q as the MFMA B operand: lane (g, c) holds Q[head 16*nb + c][32*ks + 8g .. +7]
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int head_in_group = w.hb * kHB + 16 * nb + c;
+    const bool head_ok = head_in_group < a.G;
+    const int head = w.kvh * a.G + head_in_group;
     const char* qp = (const char*)a.q + ((int64_t)w.b * a.sq_b + (int64_t)head * a.sq_h) * 2;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 z = {0u, 0u, 0u, 0u};
-      qop[ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
+      qop[nb][ks] = head_ok ? *(const u32x4*)(qp + (32 * ks + 8 * g) * 2) : z;
     }
   }
 
@@ -100,11 +105,15 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
     }
   };
 
-  float m = -INFINITY;
-  float l = 0.f;
-  f32x4 acc[8];  // acc[j][i] = O[head c][dim 16*(r & 7) + 8*(r >> 3) + j], r = 4g + i
+  float m[NB], l[NB];
+  f32x4 acc[NB][8];  // acc[nb][j][i] = O[head 16*nb + c][dim 16*(r & 7) + 8*(r >> 3) + j], r = 4g + i
 #pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int nb = 0; nb < NB; ++nb) {
+    m[nb] = -INFINITY;
+    l[nb] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[nb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   int pg_next = 0, slot_next = 0;
   int rv_cur = 0;  // flat rows of the tile whose V is still to be requested
@@ -124,9 +133,11 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- S^T = K . Q^T, four 16-token sub-tiles
-    f32x4 s[4];
+    f32x4 s[NB][4];
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) s[nb][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
@@ -135,37 +146,42 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
         const uint32_t k0 = kk[0], k1 = kk[1];
         u32x4 ak = {Mma<T>::from_fp8(k0, false), Mma<T>::from_fp8(k0, true), Mma<T>::from_fp8(k1, false),
                     Mma<T>::from_fp8(k1, true)};
-        s[tt] = Mma<T>::run(ak, qop[ks], s[tt]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) s[nb][tt] = Mma<T>::run(ak, qop[nb][ks], s[nb][tt]);
       }
     }
-    // ---- online softmax: x[4*tt + i] <-> token 16*tt + 4g + i, head c
-    float x[16];
+    // ---- online softmax: x[4*tt + i] <-> token 16*tt + 4g + i, head 16*nb + c
     const int n0 = w.start + t * kTile;
     const bool full = n0 + kTile <= w.end;
+    u32x4 pop[NB][2];  // P^T B operands: block kb, element e <-> token 16*(2kb + e/4) + 4g + e%4
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
+    for (int nb = 0; nb < NB; ++nb) {
+      float x[16];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v = s[tt][i];
-        if (SOFTCAP) {
-          v = fd_softcap(v * kq_scale, a.soft_cap, inv_cap) * FD_LOG2E;
-        } else {
-          v *= scale2;
+      for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = s[nb][tt][i];
+          if (SOFTCAP) {
+            v = fd_softcap(v * kq_scale, a.soft_cap, inv_cap) * FD_LOG2E;
+          } else {
+            v *= scale2;
+          }
+          x[4 * tt + i] = (full || n0 + 16 * tt + 4 * g + i < w.end) ? v : -INFINITY;
         }
-        x[4 * tt + i] = (full || n0 + 16 * tt + 4 * g + i < w.end) ? v : -INFINITY;
       }
+      bool moved;
+      const float alpha = fd_softmax_step(x, m[nb], l[nb], moved);
+      if (moved) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[nb][j] *= alpha;
+      }
+#pragma unroll
+      for (int kblk = 0; kblk < 2; ++kblk)
+#pragma unroll
+        for (int q2 = 0; q2 < 4; ++q2)
+          pop[nb][kblk][q2] = Mma<T>::pack(x[8 * kblk + 2 * q2], x[8 * kblk + 2 * q2 + 1]);
     }
-    bool moved;
-    const float alpha = fd_softmax_step(x, m, l, moved);
-    if (moved) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] *= alpha;
-    }
-    u32x4 pop[2];  // P^T B operands: block kb, element e <-> token 16*(2kb + e/4) + 4g + e%4
-#pragma unroll
-    for (int kblk = 0; kblk < 2; ++kblk)
-#pragma unroll
-      for (int q2 = 0; q2 < 4; ++q2) pop[kblk][q2] = Mma<T>::pack(x[8 * kblk + 2 * q2], x[8 * kblk + 2 * q2 + 1]);
 
     // ---- V: dequantise, transpose 8 tokens x 8 dims per block, O^T += V^T . P^T
 #pragma unroll
@@ -191,7 +207,8 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
         u32x4 vop;
 #pragma unroll
         for (int q2 = 0; q2 < 4; ++q2) vop[q2] = __builtin_amdgcn_perm(cv[2 * q2 + 1][j >> 1], cv[2 * q2][j >> 1], sel);
-        acc[j] = Mma<T>::run(vop, pop[kblk], acc[j]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb][j] = Mma<T>::run(vop, pop[nb][kblk], acc[nb][j]);
       }
     }
   };
@@ -211,22 +228,27 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
   }
 
   // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
   wave_lds_fence();
   float* part = (float*)kb;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = 4 * g + i;
-    const int dim0 = 16 * (r & 7) + 8 * (r >> 3);
-    f32x4 lo = {acc[0][i], acc[1][i], acc[2][i], acc[3][i]};
-    f32x4 hi = {acc[4][i], acc[5][i], acc[6][i], acc[7][i]};
-    *(f32x4*)(part + c * kD + dim0) = lo;
-    *(f32x4*)(part + c * kD + dim0 + 4) = hi;
-  }
-  if (g == 0) {
-    part[kHB * kD + c] = m;
-    part[kHB * kD + kHB + c] = l;
+  for (int nb = 0; nb < NB; ++nb) {
+    float lsum = l[nb];
+    lsum += __shfl_xor(lsum, 16);
+    lsum += __shfl_xor(lsum, 32);
+    const int h = 16 * nb + c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * g + i;
+      const int dim0 = 16 * (r & 7) + 8 * (r >> 3);
+      f32x4 lo = {acc[nb][0][i], acc[nb][1][i], acc[nb][2][i], acc[nb][3][i]};
+      f32x4 hi = {acc[nb][4][i], acc[nb][5][i], acc[nb][6][i], acc[nb][7][i]};
+      *(f32x4*)(part + h * kD + dim0) = lo;
+      *(f32x4*)(part + h * kD + dim0 + 4) = hi;
+    }
+    if (g == 0) {
+      part[kHB * kD + h] = m[nb];
+      part[kHB * kD + kHB + h] = lsum;
+    }
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
@@ -236,19 +258,26 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_kernel(const SplitArgs 
 
 }  // namespace
 
+template <typename T>
+static auto pick_kernel(bool soft_cap, int nb) -> void (*)(const SplitArgs) {
+  if (nb == 2) return soft_cap ? fd_split_mfma_fp8_kernel<T, true, 2> : fd_split_mfma_fp8_kernel<T, false, 2>;
+  return soft_cap ? fd_split_mfma_fp8_kernel<T, true, 1> : fd_split_mfma_fp8_kernel<T, false, 1>;
+}
+
 int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap) {
   const dim3 grid = fd_split_grid(a);
   const unsigned block = 64u * waves;
-  size_t lds = (size_t)waves * kWaveLds;
+  const int nb = a.hbsz > 16 ? 2 : 1;   // a.hbsz = query heads per head block: up to 16, or up to 32 (two per wave)
+  size_t lds = (size_t)waves * wave_lds(nb);
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
-    const size_t need = (size_t)(a.S + a.num_extra) * kHB * 4;
+    const size_t need = (size_t)(a.S + a.num_extra) * 16 * nb * 4;
     if (need > lds) lds = need;
   }
   void (*kern)(const SplitArgs) = nullptr;
   if (q_dtype == FD_BF16) {
-    kern = soft_cap ? fd_split_mfma_fp8_kernel<__bf16, true> : fd_split_mfma_fp8_kernel<__bf16, false>;
+    kern = pick_kernel<__bf16>(soft_cap, nb);
   } else if (q_dtype == FD_F16) {
-    kern = soft_cap ? fd_split_mfma_fp8_kernel<_Float16, true> : fd_split_mfma_fp8_kernel<_Float16, false>;
+    kern = pick_kernel<_Float16>(soft_cap, nb);
   } else {
     return FD_ERR_UNSUPPORTED;
   }
