@@ -55,8 +55,12 @@ bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
 
 // Query-head slots of one head block of the MFMA kernels: 16 (one MFMA column block per wave), or 32 where the kernel
 // serves two column blocks per wave from one pass over K and V and the group is large enough to use them.
+int env_int(const char* name);
+
 int mfma_head_block(int head_dim, int group, int kv_dtype) {
   if (head_dim != 128) return 16;
+  static const int forced = env_int("FD_HEAD_BLOCK");   // tuning override for experiments: 16 or 32
+  if (forced == 16 || forced == 32) return forced;
   if (kv_dtype == FD_F16 || kv_dtype == FD_BF16) return group > 16 ? 32 : 16;
   // fp8: two sibling waves of 16 heads each still beat one two-block wave (G = 32: 47.3 vs 52.1 us on config 2's
   // shape); beyond that two two-block waves beat four sibling waves (G = 64: 62.5 vs 77.0 us)
@@ -93,7 +97,8 @@ constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged b
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
 
 // Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
-// split) where the caller leaves the choice to the library) and FD_HEADS_PER_BLOCK (members per workgroup).
+// split) where the caller leaves the choice to the library), FD_HEADS_PER_BLOCK (members per workgroup) and
+// FD_HEAD_BLOCK (16 or 32 query heads per wave in the head_dim-128 kernels).
 int env_int(const char* name) {
   const char* e = getenv(name);
   return e ? atoi(e) : 0;
