@@ -413,11 +413,45 @@ def test_fp8_decode_matches_oracle_on_dequantised_cache(fd, num_heads, D):
     ref, ref_lse = oracle_decode(wl)
     assert_out_close(out, ref)
     assert_lse_close(lse, ref_lse)
-    if D != 64:   # head_dim 128 / 256 have an MFMA and a VALU kernel: force each
-        for path, extra in (("valu", {}), ("mfma", dict(waves_per_block=4, plan_splits=False))):
-            out_p, lse_p = run_decode(fd, wl, path=path, **extra)
-            assert_out_close(out_p, ref)
-            assert_lse_close(lse_p, ref_lse)
+    for path, extra in (("valu", {}), ("mfma", dict(waves_per_block=4, plan_splits=False))):   # force each kernel
+        out_p, lse_p = run_decode(fd, wl, path=path, **extra)
+        assert_out_close(out_p, ref)
+        assert_lse_close(lse_p, ref_lse)
+
+
+def test_fp8_d64_dequant_table_and_soft_cap(fd):
+    """All byte patterns through the head_dim-64 fp8 kernels (kv_len == 1: out == dequantised V[0], exact), and the
+    soft cap with a 40-head group over ragged lengths."""
+    tab = torch.from_numpy(oracle.fp8_e4m3fn_decode_table())
+    bytes_ = torch.arange(256, dtype=torch.uint8)
+    bytes_[0x7f] = 0
+    bytes_[0xff] = 0x80
+    Hkv, D = 4, 64
+    v = bytes_.view(1, 1, Hkv, D).clone()
+    k = torch.full_like(v, 0x38)  # 1.0
+    k_scale = torch.tensor([0.5, 2.0, 1.0, 0.25])
+    v_scale = torch.tensor([0.25, 3.0, 1.0, 0.5])
+    q = torch.ones(1, 8, D, dtype=torch.float16)
+    bt = torch.tensor([[0]], dtype=torch.int32)
+    for path in ("valu", "mfma"):
+        lse = torch.empty(1, 8, dtype=torch.float32, device=DEV)
+        out = fd.gqa_fwd_batch_decode(q.to(DEV), k.to(DEV), v.to(DEV), None, [1],
+                                      torch.tensor([1], dtype=torch.int32, device=DEV), bt.to(DEV), 0.125,
+                                      output_combine=torch.empty(1, 8, D, dtype=torch.float32, device=DEV),
+                                      lse_out=lse, k_scale=k_scale.to(DEV), v_scale=v_scale.to(DEV), path=path)
+        torch.cuda.synchronize()
+        out = out.cpu()
+        for h in range(8):
+            kvh = h // 2
+            assert torch.equal(out[0, h], tab[v[0, 0, kvh].long()] * v_scale[kvh]), (path, h)
+            assert math.isclose(lse[0, h].item(), 0.125 * 64 * k_scale[kvh].item(), rel_tol=1e-6)
+    wl = fd.utils.make_paged_workload("fp8_d64_cap", [700, 129, 31, 2050], 80, 2, 64, 1, torch.float16, 32, seed=63,
+                                      soft_cap=30.0, fp8_kv=True)
+    ref, ref_lse = oracle_decode(wl)
+    for kw in (dict(), dict(path="mfma", waves_per_block=8, plan_splits=False), dict(fuse_combine=True)):
+        out, lse = run_decode(fd, wl, **kw)
+        assert_out_close(out, ref)
+        assert_lse_close(lse, ref_lse)
 
 
 def test_fp8_d256_dequant_table_and_soft_cap(fd):

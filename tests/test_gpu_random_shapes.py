@@ -33,7 +33,18 @@ def _case(i):
 
 @pytest.mark.parametrize("i", range(CASES))
 def test_random_shape(fd, i):
-    c = _case(i)
+    _check_case(fd, _case(i), i)
+
+
+@pytest.mark.parametrize("i", range(40))
+def test_random_shape_fp8_head_dim_64(fd, i):
+    """The same sweep pinned to 64-byte fp8 rows, which have an MFMA kernel of their own (K and V both through LDS)."""
+    c = _case(500 + i)
+    c.update(D=64, kind="fp8")
+    _check_case(fd, c, 500 + i)
+
+
+def _check_case(fd, c, i):
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp8": torch.bfloat16, "fp32": torch.float32}[c["kind"]]
     wl = fd.utils.make_paged_workload(f"rand{i}", c["lens"], c["Hq"], c["Hkv"], c["D"], c["P"], dtype, c["kv_split"],
                                       seed=7000 + i, soft_cap=c["soft_cap"], fp8_kv=c["kind"] == "fp8", pool_slack_pages=3)

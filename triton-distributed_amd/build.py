@@ -20,7 +20,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 BUILD = os.path.join(PKG_DIR, "_build")
 LIB_NAME = "libflash_decode_gfx950.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ["fd_api.hip", "fd_split_mfma.hip", "fd_split_mfma_fp8.hip", "fd_split_mfma_fp8_d256.hip", "fd_split_mfma_d256.hip", "fd_split_mfma_d64.hip", "fd_split_valu.hip", "fd_combine.hip",
+SOURCES = ["fd_api.hip", "fd_split_mfma.hip", "fd_split_mfma_fp8.hip", "fd_split_mfma_fp8_d256.hip", "fd_split_mfma_fp8_d64.hip", "fd_split_mfma_d256.hip", "fd_split_mfma_d64.hip", "fd_split_valu.hip", "fd_combine.hip",
            "fd_kv_append.hip"]
 HEADERS = [os.path.join(CSRC, "fd_common.h"), os.path.join(CSRC, "fd_mma.h"),
            os.path.join(os.path.dirname(PKG_DIR), "include", "flash_decode.h")]

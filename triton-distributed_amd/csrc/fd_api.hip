@@ -42,15 +42,13 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
   *shift = k;
 }
 
-// Shapes the MFMA split kernels are built for: head_dim 128 or 256 with a 16-bit or fp8-e4m3 cache, head_dim 64 with
-// a 16-bit cache; any GQA group (blocks of 16 query heads, the last one padded: even with one
+// Shapes the MFMA split kernels are built for: head_dim 64, 128 or 256 with a 16-bit or fp8-e4m3 cache; any GQA group (blocks of 16 query heads, the last one padded: even with one
 // query head per KV head the MFMA kernels stream faster than the VALU kernel, 46.1 vs 50.2 us on config 2's shape as MHA,
 // 46.1 vs 78.9 us with 3 query heads per KV head).
 bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
   const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
-  const bool dim_ok = ((head_dim == 128 || head_dim == 256) && (kv16 || kv_dtype == FD_FP8_E4M3)) || (head_dim == 64 && kv16);
   (void)group;
-  return dim_ok;
+  return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (kv16 || kv_dtype == FD_FP8_E4M3);
 }
 
 // Query-head slots of one head block of the MFMA kernels: 16 (one MFMA column block per wave), or 32 where the kernel
@@ -67,6 +65,9 @@ int mfma_head_block(int head_dim, int group, int kv_dtype) {
   if (kv_dtype == FD_FP8_E4M3) return group > 32 ? 32 : 16;
   return 16;
 }
+
+// Whether the fp8 head_dim-64 kernel can serve two adjacent KV heads per wave (given contiguous rows).
+bool fp8_d64_pairs(int group, int kv_heads) { return group <= 16 && kv_heads % 2 == 0; }
 
 // fd_params.split_adapt: 0, or a power of two together with a split alignment and a power-of-two split count.
 int check_split_adapt(const char* fn, const fd_params* p) {
@@ -233,17 +234,24 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs head_dim 128 / 256 (or 64 with a 16-bit cache), a 16-bit query with a KV cache "
-                "of the same dtype or fp8-e4m3, and 16-byte aligned q rows", fn);
+                "%s: MFMA path needs a 16-bit query with a KV cache of the same dtype or fp8-e4m3, and 16-byte aligned "
+                "q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
 
+  // fp8 rows of head_dim 64 are half a cache line: where two adjacent KV heads' rows are one contiguous 128 bytes,
+  // a wave of the MFMA kernel serves both, and the pair is presented to the kernel as one KV head with 2 G query heads
+  const bool pair = use_mfma && kv_fp8 && D == 64 && fp8_d64_pairs(G, p->kv_heads) && stride_k_h == 64 && stride_v_h == 64;
+  if (pair) {
+    a.Hkv = p->kv_heads / 2;
+    a.G = 2 * G;
+  }
   int tile;
   if (use_mfma) {
-    const int hb = mfma_head_block(D, G, p->kv_dtype);
-    a.hbsz = G < hb ? G : hb;
-    a.nhb = (G + hb - 1) / hb;
+    const int hb = pair ? 32 : mfma_head_block(D, G, p->kv_dtype);
+    a.hbsz = a.G < hb ? a.G : hb;
+    a.nhb = (a.G + hb - 1) / hb;
     tile = kv_fp8 ? (D == 256 ? 32 : 64) : (D == 64 ? 64 : (D == 256 ? 16 : 32));
   } else {
     a.hbsz = G >= 3 ? 4 : G;
@@ -257,9 +265,12 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : a.S;
   const int64_t wgs = (int64_t)batch * busy_splits * a.Hkv * a.nhb;
   // the two-block MFMA kernel needs the register file of a whole SIMD per wave: workgroups of at most 4 waves
-  const int max_waves = use_mfma && a.hbsz > 16 ? 4 : 8;
+  const int max_waves = use_mfma && (a.hbsz > 16 || pair) ? 4 : 8;
+  // the fp8 head_dim-64 kernel keeps 8 KB in flight per wave with one KV head per wave, like the VALU kernel;
+  // the other MFMA kernels 16 KB
+  const int64_t wave_target = use_mfma && !(kv_fp8 && D == 64 && !pair) ? kTargetWaves : kTargetWavesValu;
   int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
-                                 : choose_waves(wgs, max_tok_split, tile, use_mfma ? kTargetWaves : kTargetWavesValu, max_waves);
+                                 : choose_waves(wgs, max_tok_split, tile, wave_target, max_waves);
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
@@ -275,7 +286,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
       a.member_hb = 1;
     }
   } else if (use_mfma && !fuse) {
-    a.hpw = choose_heads_per_group(a.Hkv, D * kvsz, waves, wgs, max_waves);
+    a.hpw = choose_heads_per_group(a.Hkv, D * kvsz * (pair ? 2 : 1), waves, wgs, max_waves);
   }
   a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / a.hpw * a.nhb;
   a.nsub = waves;
@@ -283,7 +294,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   // fuse the combine into the split kernel's tail when a ticket buffer is there and the LSEs fit in LDS
   if (fuse) {  // the fused tail exchanges fp32 partials only
-    const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (use_mfma && a.hbsz < 16 ? 16 : a.hbsz) * 4;
+    const size_t lse_lds = (size_t)(a.S + tail->num_extra) * (pair ? 32 : use_mfma && a.hbsz < 16 ? 16 : a.hbsz) * 4;
     if (lse_lds <= kMaxLds / 2) {
       a.tickets = tail->tickets; a.fout = tail->out; a.flse = tail->lse_out;
       a.extra_out = tail->extra_out; a.extra_lse = tail->extra_lse;
@@ -296,6 +307,8 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   int rc;
   if (use_mfma && kv_fp8 && D == 256) {
     rc = fd_launch_split_mfma_fp8_d256((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
+  } else if (use_mfma && kv_fp8 && D == 64) {
+    rc = fd_launch_split_mfma_fp8_d64((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f, pair ? 2 : 1);
   } else if (use_mfma && kv_fp8) {
     rc = fd_launch_split_mfma_fp8((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
   } else if (use_mfma && D == 64) {
@@ -406,7 +419,10 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
   const bool mfma = mfma_shape_ok(p->head_dim, G, p->kv_dtype) && p->path != FD_PATH_VALU;
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
-  const int64_t groups = (int64_t)batch * p->kv_heads * nhb;        // (KV head, head block) pairs per split
+  // fp8 rows of head_dim 64: two KV heads per wave (the usual cache layout has their rows side by side)
+  const bool pair = mfma && p->kv_dtype == FD_FP8_E4M3 && p->head_dim == 64 && fp8_d64_pairs(G, p->kv_heads);
+  const int kv_units = pair ? p->kv_heads / 2 : p->kv_heads;
+  const int64_t groups = (int64_t)batch * kv_units * nhb;        // (KV head, head block) pairs per split
   const int64_t max_tokens = planned_tokens(p);
   int64_t s = 1;
   if (mfma) {
@@ -417,9 +433,9 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
       for (int h = 4; h > 1; --h)
         if (nhb % h == 0) { members = h; break; }
     } else {
-      const int row_bytes = p->head_dim * dtype_size(p->kv_dtype);
+      const int row_bytes = p->head_dim * dtype_size(p->kv_dtype) * (pair ? 2 : 1);
       members = row_bytes > 0 && row_bytes < 512 ? 512 / row_bytes : 1;
-      while (members > 1 && p->kv_heads % members != 0) members >>= 1;
+      while (members > 1 && kv_units % members != 0) members >>= 1;
     }
     while (s * groups < kMinWorkgroups * members) s <<= 1;
     // (2) ... and a whole number of workgroups per CU, or at least four, while a split of a full-length sequence
