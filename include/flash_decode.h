@@ -53,8 +53,8 @@ typedef enum fd_dtype {
 } fd_dtype;
 
 typedef enum fd_path {
-  FD_PATH_AUTO = 0,         /* MFMA for head_dim 128 / 256 (16-bit or fp8 KV) and 64
-                               (16-bit KV) with a 16-bit query; else VALU          */
+  FD_PATH_AUTO = 0,         /* MFMA for a 16-bit query with a KV cache of the same
+                               dtype or fp8-e4m3; else VALU                        */
   FD_PATH_VALU = 1,         /* force the VALU dot-product kernel                   */
   FD_PATH_MFMA = 2          /* force MFMA; FD_ERR_UNSUPPORTED if not applicable    */
 } fd_path;
