@@ -328,6 +328,45 @@ def test_strided_inputs(fd):
     assert_lse_close(lse, ref_lse)
 
 
+@pytest.mark.parametrize("layout", ["fused_kv", "padded_heads"])
+def test_strided_fp8_head_dim_64(fd, layout):
+    """fp8 caches of 64-byte rows as views: K and V as head-slices of one fused tensor (rows of two adjacent KV heads
+    still side by side: a wave may serve both), and as the first 64 bytes of 128-byte head slots (they are not)."""
+    gen = torch.Generator(device="cpu").manual_seed(43)
+    Hkv, G, D = 4, 6, 64
+    raw = torch.randint(0, 256, (200, 16, 2 * Hkv, 2 * D), generator=gen, dtype=torch.uint8)
+    raw[(raw & 0x7f) == 0x7f] = 0x11          # no NaN patterns
+    raw[(raw & 0x78) == 0x78] &= 0xb7         # keep magnitudes moderate
+    if layout == "fused_kv":
+        big = raw[..., :D].contiguous()                      # [pages, P, 2*Hkv, 64]
+        k, v = big[:, :, :Hkv], big[:, :, Hkv:]
+    else:
+        k, v = raw[:, :, :Hkv, :D], raw[:, :, Hkv:, :D]      # head stride 128
+    assert not k.is_contiguous() and k.stride(-2) == (D if layout == "fused_kv" else 2 * D)
+    q = torch.randn(3, Hkv * G, D, generator=gen).to(torch.float16)
+    kv_lens = [700, 1, 2049]
+    bt = torch.randint(0, 200, (3, 129), generator=gen, dtype=torch.int32)
+    k_scale = torch.tensor([0.02, 0.01, 0.03, 0.015])
+    v_scale = torch.tensor([0.5, 1.0, 0.25, 2.0])
+    tab = torch.from_numpy(oracle.fp8_e4m3fn_decode_table())
+    ref, ref_lse = oracle.ref_paged_attn_lse(q.float(), tab[k.long()] * k_scale[None, None, :, None],
+                                             tab[v.long()] * v_scale[None, None, :, None], kv_lens, bt, D ** -0.5)
+    if layout == "fused_kv":
+        gbig = big.to(DEV)
+        gk, gv = gbig[:, :, :Hkv], gbig[:, :, Hkv:]
+    else:
+        graw = raw.to(DEV)
+        gk, gv = graw[:, :, :Hkv, :D], graw[:, :, Hkv:, :D]
+    for path in ("auto", "valu"):
+        lse = torch.empty(3, Hkv * G, dtype=torch.float32, device=DEV)
+        out = fd.gqa_fwd_batch_decode(q.to(DEV), gk, gv, None, [1] * 3, torch.tensor(kv_lens, dtype=torch.int32, device=DEV),
+                                      bt.to(DEV), D ** -0.5, lse_out=lse, k_scale=k_scale.to(DEV), v_scale=v_scale.to(DEV),
+                                      path=path)
+        torch.cuda.synchronize()
+        assert_out_close(out.cpu(), ref)
+        assert_lse_close(lse.cpu(), ref_lse)
+
+
 # ---- caller-supplied partial buffers in the reference layout [B, Hq, S, Dv+1]
 @pytest.mark.parametrize("mid_dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("num_heads", [(32, 8), (4, 4)])
