@@ -182,8 +182,12 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
         } else {
           v *= scale2;
         }
-        const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
-        x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
+        x[i] = v;
+      }
+      if (!full) {   // only the last tile of a range has tokens to mask (wave-uniform branch)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (n0 + 4 * g + (i & 3) + 16 * (i >> 2) >= w.end) x[i] = -INFINITY;
       }
       bool moved;
       const float alpha = fd_softmax_step(x, m[nb], l[nb], moved);

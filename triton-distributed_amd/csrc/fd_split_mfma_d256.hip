@@ -155,7 +155,12 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d256_kernel(const SplitAr
       } else {
         v *= scale2;
       }
-      x[i] = (full || n0 + 4 * g + i < w.end) ? v : -INFINITY;
+      x[i] = v;
+    }
+    if (!full) {   // only the last tile of a range has tokens to mask (wave-uniform branch)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n0 + 4 * g + i >= w.end) x[i] = -INFINITY;
     }
     bool moved;
     const float alpha = fd_softmax_step(x, m, l, moved);

@@ -141,8 +141,13 @@ __global__ void __launch_bounds__(512) fd_split_mfma16_d64_kernel(const SplitArg
         } else {
           v *= scale2;
         }
-        x[4 * tt + i] = (full || n0 + 16 * tt + 4 * g + i < w.end) ? v : -INFINITY;
+        x[4 * tt + i] = v;
       }
+    }
+    if (!full) {   // only the last tile of a range has tokens to mask (wave-uniform branch)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        if (n0 + 16 * (e >> 2) + 4 * g + (e & 3) >= w.end) x[e] = -INFINITY;
     }
     bool moved;
     const float alpha = fd_softmax_step(x, m, l, moved);

@@ -143,8 +143,12 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
       } else {
         v *= scale2;
       }
-      const int tau = 4 * g + (i & 3) + 16 * (i >> 2);
-      x[i] = (full || n0 + tau < w.end) ? v : -INFINITY;
+      x[i] = v;
+    }
+    if (!full) {   // only the last tile of a range has tokens to mask (wave-uniform branch)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (n0 + 4 * g + (i & 3) + 16 * (i >> 2) >= w.end) x[i] = -INFINITY;
     }
     bool moved;
     const float alpha = fd_softmax_step(x, m, l, moved);
