@@ -131,6 +131,10 @@ int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_
   if (env_heads() > 0) h = env_heads();
   if (h < 1) h = 1;
   while (h > 1 && (kv_heads % h != 0 || h * waves > max_waves || head_splits / h < kMinWorkgroups)) h >>= 1;
+  // Between one and one and a half workgroups per CU the busiest CUs hold two workgroups of h members; with half the
+  // members they hold three of h / 2 (measured 3 - 7 % faster there: B = 5 x 5000 tokens 22.4 -> 20.8 us)
+  const int64_t nwg = head_splits / h;
+  if (h > 1 && nwg > kMinWorkgroups && 2 * nwg <= 3 * kMinWorkgroups) h >>= 1;
   return h;
 }
 
