@@ -204,6 +204,12 @@ def test_split_plan_policy(fd):
     assert plan(8, 32, 8, 32, 512, D=256) == 4     # head_dim 256: 512-byte rows, no sibling heads -> 256 workgroups
     assert plan(8, 32, 8, 32, 512, D=64) == 16     # head_dim 64: four sibling heads per workgroup
     assert plan(8, 8, 8, 32, 512) == 8             # MHA runs on the MFMA kernels too
+    # fp8 rows of head_dim 64: a wave takes two adjacent KV heads (4 pairs, all in one workgroup) ...
+    assert plan(64, 32, 8, 32, 256, kv=L.FD_FP8_E4M3, D=64) == 4
+    assert plan(8, 32, 8, 64, 512, kv=L.FD_FP8_E4M3, D=64) == 32
+    # ... but not with an odd number of KV heads or more than 16 query heads per KV head
+    assert plan(64, 24, 3, 32, 256, kv=L.FD_FP8_E4M3, D=64) == 4     # 192 single heads: 2 splits = 1.5 per CU -> 4
+    assert plan(64, 40, 2, 32, 256, kv=L.FD_FP8_E4M3, D=64) == 2
     assert plan(8, 8, 8, 32, 512, kv=L.FD_F32) == 8  # VALU path (fp32 cache): 2048 waves with 4 waves per (head, split)
     assert plan(2, 8, 8, 32, 512) == 32
     assert plan(3, 32, 8, 32, 512) == 32           # 21.3 -> the next power of two
