@@ -42,19 +42,25 @@ void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
   *shift = k;
 }
 
-// Shapes the MFMA split kernels are built for: head_dim 64, 128 or 256 with a 16-bit or fp8-e4m3 cache; any GQA group (blocks of 16 query heads, the last one padded: even with one
-// query head per KV head the MFMA kernels stream faster than the VALU kernel, 46.1 vs 50.2 us on config 2's shape as MHA,
-// 46.1 vs 78.9 us with 3 query heads per KV head).
-bool mfma_shape_ok(int head_dim, int group, int kv_dtype) {
+// Shapes the MFMA split kernels are built for: head_dim 64, 128 or 256 with a 16-bit or fp8-e4m3 cache; any GQA
+// group (blocks of 16 query heads, the last one padded: even with one query head per KV head the MFMA kernels stream
+// faster than the VALU kernel, 46.1 vs 50.2 us on config 2's shape as MHA, 46.1 vs 78.9 us with 3 query heads per
+// KV head).
+bool mfma_shape_ok(int head_dim, int kv_dtype) {
   const bool kv16 = kv_dtype == FD_F16 || kv_dtype == FD_BF16;
-  (void)group;
   return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (kv16 || kv_dtype == FD_FP8_E4M3);
+}
+
+// Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
+// split) where the caller leaves the choice to the library), FD_HEADS_PER_BLOCK (members per workgroup) and
+// FD_HEAD_BLOCK (16 or 32 query heads per wave in the head_dim-128 kernels).
+int env_int(const char* name) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : 0;
 }
 
 // Query-head slots of one head block of the MFMA kernels: 16 (one MFMA column block per wave), or 32 where the kernel
 // serves two column blocks per wave from one pass over K and V and the group is large enough to use them.
-int env_int(const char* name);
-
 int mfma_head_block(int head_dim, int group, int kv_dtype) {
   if (head_dim != 128) return 16;
   static const int forced = env_int("FD_HEAD_BLOCK");   // tuning override for experiments: 16 or 32
@@ -97,13 +103,6 @@ constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
 
-// Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
-// split) where the caller leaves the choice to the library), FD_HEADS_PER_BLOCK (members per workgroup) and
-// FD_HEAD_BLOCK (16 or 32 query heads per wave in the head_dim-128 kernels).
-int env_int(const char* name) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : 0;
-}
 int env_waves() {
   static const int v = env_int("FD_WAVES_PER_BLOCK");
   return v;
@@ -232,7 +231,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
   const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
-  const bool mfma_ok = mfma_shape_ok(D, G, p->kv_dtype) && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
+  const bool mfma_ok = mfma_shape_ok(D, p->kv_dtype) && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
                        aligned16(q) && stride_q_bs % 8 == 0 && stride_q_h % 8 == 0;
   bool use_mfma = mfma_ok;
   if (p->path == FD_PATH_VALU) use_mfma = false;
@@ -420,7 +419,7 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
       p->page_size <= 0 || p->max_pages_per_seq <= 0)
     return fail(FD_ERR_INVALID_ARG, "%s: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0", fn);
   const int G = p->q_heads / p->kv_heads;
-  const bool mfma = mfma_shape_ok(p->head_dim, G, p->kv_dtype) && p->path != FD_PATH_VALU;
+  const bool mfma = mfma_shape_ok(p->head_dim, p->kv_dtype) && p->path != FD_PATH_VALU;
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
   // fp8 rows of head_dim 64: two KV heads per wave (the usual cache layout has their rows side by side)
