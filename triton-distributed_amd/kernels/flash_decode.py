@@ -100,30 +100,43 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
                  waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0,
                  max_kv_len=0) -> FdParams:
-    p = FdParams()
-    p.q_heads = q.shape[1]
-    p.kv_heads = k_cache.shape[2]
-    p.head_dim = q.shape[2]
-    p.page_size = k_cache.shape[1]
-    p.num_splits = kv_split
-    p.num_pages = k_cache.shape[0]
-    p.max_pages_per_seq = block_table.shape[1]
-    p.q_dtype = fd_dtype_of(q)
-    p.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
-    p.mid_dtype = mid_dtype
-    p.out_dtype = out_dtype
-    p.soft_cap = float(soft_cap or 0.0)
-    p.k_scale = k_scale.data_ptr() if k_scale is not None else None
-    p.v_scale = v_scale.data_ptr() if v_scale is not None else None
-    p.path = _PATHS[path]
-    p.waves_per_block = waves_per_block
-    p.seq_order_lens = seq_order_lens.data_ptr() if seq_order_lens is not None else None
-    p.split_align = split_align
-    p.split_adapt = split_adapt
-    p.seq_order_items = seq_order_items
-    p.max_kv_len = max_kv_len
+    # the scalar fields are the same from step to step: filled once per combination, copied per call
+    key = (q.shape, k_cache.shape, block_table.shape[1], q.dtype, k_cache.dtype, k_scale is not None, kv_split, soft_cap,
+           mid_dtype, out_dtype, path, waves_per_block, split_align, split_adapt, seq_order_items, max_kv_len)
+    template = _PARAMS_CACHE.get(key)
+    if template is None:
+        t = FdParams()
+        t.q_heads = q.shape[1]
+        t.kv_heads = k_cache.shape[2]
+        t.head_dim = q.shape[2]
+        t.page_size = k_cache.shape[1]
+        t.num_splits = kv_split
+        t.num_pages = k_cache.shape[0]
+        t.max_pages_per_seq = block_table.shape[1]
+        t.q_dtype = fd_dtype_of(q)
+        t.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
+        t.mid_dtype = mid_dtype
+        t.out_dtype = out_dtype
+        t.soft_cap = float(soft_cap or 0.0)
+        t.path = _PATHS[path]
+        t.waves_per_block = waves_per_block
+        t.split_align = split_align
+        t.split_adapt = split_adapt
+        t.seq_order_items = seq_order_items
+        t.max_kv_len = max_kv_len
+        if len(_PARAMS_CACHE) > 4096:
+            _PARAMS_CACHE.clear()
+        template = _PARAMS_CACHE[key] = bytes(t)
+    p = FdParams.from_buffer_copy(template)
+    if k_scale is not None:
+        p.k_scale = k_scale.data_ptr()
+        p.v_scale = v_scale.data_ptr()
+    if seq_order_lens is not None:
+        p.seq_order_lens = seq_order_lens.data_ptr()
     return p
 
+
+_PARAMS_CACHE = {}   # fd_params images by their scalar fields
 
 MAX_ITEM_BATCH = 1024       # sequences fd_schedule_items ranks in one launch
 MAX_FUSED_ITEM_BATCH = 256  # ... and fd_kv_append in its trailing workgroup
@@ -179,9 +192,10 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     assert v_head_dim == k_head_dim, "the gfx950 kernels need equal K and V head dims"
     _require_cuda(q, k_cache, v_cache, kv_lens, block_table, output_split, output_combine)
     assert kv_lens.dtype == torch.int32 and block_table.dtype == torch.int32
-    assert q.stride(-1) == 1 and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+    q_st, k_st, v_st = q.stride(), k_cache.stride(), v_cache.stride()
+    assert q_st[-1] == 1 and k_st[-1] == 1 and v_st[-1] == 1
     # kv_loc = page * P + slot is a flat token index (flash_decode.py:205-206): the pool must be linear in it
-    assert k_cache.stride(0) == page_size * k_cache.stride(1) and v_cache.stride(0) == page_size * v_cache.stride(1)
+    assert k_st[0] == page_size * k_st[1] and v_st[0] == page_size * v_st[1]
     if (k_scale is None) != (v_scale is None):
         raise RuntimeError("k_scale and v_scale must be given together")
     num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
@@ -225,8 +239,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     out_cols = v_head_dim + 1 if with_lse_column else v_head_dim
     if output_combine is None:
         output_combine = torch.empty([batch, q_heads, out_cols], dtype=q.dtype, device=q.device)
-    else:
-        assert output_combine.shape[-1] >= out_cols and output_combine.stride(-1) == 1
+    oc_st = output_combine.stride()
+    assert output_combine.shape[-1] >= out_cols and oc_st[-1] == 1
 
     if seq_order_lens is not None:
         assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
@@ -271,8 +285,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), mid_ptr, lse_split_ptr,
         output_combine.data_ptr(), lse_out.data_ptr() if lse_out is not None else None, float(scale),
         block_table.data_ptr(), kv_lens.data_ptr(), batch,
-        q.stride(0), q.stride(1), k_cache.stride(-3), k_cache.stride(-2), v_cache.stride(-3), v_cache.stride(-2),
-        so_b, so_h, so_s, block_table.stride(0), output_combine.stride(0), output_combine.stride(1),
+        q_st[0], q_st[1], k_st[-3], k_st[-2], v_st[-3], v_st[-2],
+        so_b, so_h, so_s, block_table.stride(0), oc_st[0], oc_st[1],
         seq_order.data_ptr() if seq_order is not None else None,
         FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
         ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra,
