@@ -367,6 +367,32 @@ def test_strided_fp8_head_dim_64(fd, layout):
         assert_lse_close(lse.cpu(), ref_lse)
 
 
+@pytest.mark.parametrize("D,dtype", [(128, torch.bfloat16), (64, torch.float16), (256, torch.bfloat16)])
+@pytest.mark.parametrize("shape", ["ramp", "steps", "falling"])
+def test_scores_that_keep_growing(fd, D, dtype, shape):
+    """The kernels rescale their accumulators only when the running maximum has grown by more than 2^8 since the last
+    rescale.  Scores that creep up by a fraction of that per tile (ramp), jump far beyond it (steps) or only fall
+    must all give the oracle's output and LSE."""
+    gen = torch.Generator(device="cpu").manual_seed(77)
+    Hq, Hkv, P, n = 8, 2, 16, 3000
+    pages = -(-n // P)
+    pos = torch.arange(pages * P, dtype=torch.float32)
+    level = {"ramp": pos / n * 60.0, "steps": (pos // 700) * 25.0, "falling": (n - pos) / n * 60.0}[shape]
+    # q = 1/sqrt(D) in every dim and k[token] = level / sqrt(D) + noise: score = scale * (level + noise . q)
+    q = torch.full((1, Hq, D), D ** -0.5).to(dtype)
+    k = (level.view(pages, P, 1, 1) * D ** -0.5 + 0.05 * torch.randn(pages, P, Hkv, D, generator=gen)).to(dtype)
+    v = torch.randn(pages, P, Hkv, D, generator=gen).to(dtype)
+    bt = torch.arange(pages, dtype=torch.int32).view(1, pages)
+    ref, ref_lse = oracle.ref_paged_attn_lse(q.float(), k.float(), v.float(), [n], bt, 1.0)
+    for kv_split in (1, 4, -1):
+        lse = torch.empty(1, Hq, dtype=torch.float32, device=DEV)
+        out = fd.gqa_fwd_batch_decode(q.to(DEV), k.to(DEV), v.to(DEV), None, [1], torch.tensor([n], dtype=torch.int32, device=DEV),
+                                      bt.to(DEV), 1.0, kv_split=kv_split, lse_out=lse)
+        torch.cuda.synchronize()
+        assert_out_close(out.cpu(), ref)
+        assert_lse_close(lse.cpu(), ref_lse)
+
+
 # ---- caller-supplied partial buffers in the reference layout [B, Hq, S, Dv+1]
 @pytest.mark.parametrize("mid_dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("num_heads", [(32, 8), (4, 4)])

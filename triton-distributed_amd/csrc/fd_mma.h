@@ -43,10 +43,11 @@ struct Mma<_Float16> {
 
 // One online-softmax step of the "lane c = head c" layout shared by the MFMA split kernels.  x[0..N) are this lane's
 // scores of head c for N tokens of the tile, in the base-2 domain, masked tokens = -inf; the four wave rows hold
-// different tokens of the same head.  Updates the running max m (identical in the four rows) and the lane's share l
-// of the running sum, replaces x by the probabilities 2^(x - m), and returns the factor the accumulators of head c
-// have to be multiplied by; moved = some lane's max moved (wave-uniform), i.e. whether that rescale is needed at all.
-// Every tile holds at least one valid token, so the new max is finite.
+// different tokens of the same head.  Updates the reference point m (identical in the four rows; at most 8 below the
+// running maximum) and the lane's share l of the running sum, replaces x by the weights 2^(x - m), and returns the
+// factor the accumulators of head c have to be multiplied by; moved = some lane's reference point moved
+// (wave-uniform), i.e. whether that rescale is needed at all.  Every tile holds at least one valid token, so the
+// new reference point is finite.
 template <int N>
 __device__ __forceinline__ float fd_softmax_step(float (&x)[N], float& m, float& l, bool& moved) {
   float t[N];   // pairwise tree: a short dependency chain
@@ -60,7 +61,12 @@ __device__ __forceinline__ float fd_softmax_step(float (&x)[N], float& m, float&
   float mx = t[0];
   mx = fmaxf(mx, __shfl_xor(mx, 16));
   mx = fmaxf(mx, __shfl_xor(mx, 32));
-  const float m_new = fmaxf(m, mx);
+  // The reference point only moves when the maximum has grown by more than kLazyMax (base-2): until then the
+  // probabilities are taken relative to the older, smaller reference (they stay below 2^kLazyMax, exact powers of two
+  // away from what the true maximum would give), and the accumulators need no rescale.  m is -inf before the first tile.
+  constexpr float kLazyMax = 8.0f;
+  const float m_top = fmaxf(m, mx);
+  const float m_new = m_top - m > kLazyMax ? m_top : m;
   const float alpha = fd_exp2(m - m_new);
   float psum = 0.f;
 #pragma unroll
