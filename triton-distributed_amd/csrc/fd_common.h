@@ -365,10 +365,11 @@ __device__ __forceinline__ int token_row(const SplitArgs& a, const int32_t* bt_r
 // part[v*stride + HB*D + h] = running max (base-2 domain), part[v*stride + HB*D + HB + h] = running
 // sum.  Wave v = member (v % hpw) + hpw * token sub-range; a member is a KV head or, for groups above 16 query
 // heads, a head block of the one KV head.  Called by every thread of the workgroup after a __syncthreads() with
-// nheads = the calling wave's head count.  scale_by_v: multiply by v_scale[kv head] (fp8 caches).
+// nheads = the calling wave's head count.  fp8 caches: the waves have already multiplied their accumulators by
+// v_scale[kv head] (a load here, between the stores, would cost its latency once per loop iteration).
 template <int HB, int D>
 __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float* part, int stride,
-                                                const WorkItem& w, int nheads, bool scale_by_v) {
+                                                const WorkItem& w, int nheads) {
   const int tid = threadIdx.x;
   const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
   constexpr int D4 = D / 4;
@@ -395,8 +396,7 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
         o += x * wgt;
       }
     }
-    const float out_scale = scale_by_v ? a.v_scale[kvh] : 1.0f;
-    float inv = L > 0.f ? out_scale / L : 0.f;
+    float inv = L > 0.f ? 1.0f / L : 0.f;
     o *= inv;
     const int head = kvh * a.G + hb * HB + h;
     const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;

@@ -6,7 +6,7 @@
 // Here K and V bytes are dequantised in registers -- v_cvt_scalef32_pk_{bf16,f16}_fp8
 // turns two e4m3 bytes into two packed 16-bit values exactly -- and fed to the same
 // 16x16x32 MFMA as the 16-bit kernel; the per-KV-head K scale is folded into the
-// softmax scale and the V scale is applied once to the finished partial.
+// softmax scale and the V scale is applied once to a wave's finished accumulators.
 //
 // Geometry per wave (lane = 16*g + m): 64-token tiles (8 KB of K and 8 KB of V).
 //   * K: 8 x global_load_dwordx4, eight whole 128-byte rows per instruction; staged
@@ -79,6 +79,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
   char* kb = smem + wave * kWaveLds;
 
   const float kq_scale = a.sm_scale * a.k_scale[w.kvh];  // K dequantisation folded into the softmax scale
+  const float v_scale = a.v_scale[w.kvh];                // V dequantisation: once, on the finished accumulators
   const float scale2 = kq_scale * FD_LOG2E;
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
@@ -247,8 +248,8 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
       const int dim0 = 16 * (r & 7) + 8 * (r >> 3);
       f32x4 lo = {acc[nb][0][i], acc[nb][1][i], acc[nb][2][i], acc[nb][3][i]};
       f32x4 hi = {acc[nb][4][i], acc[nb][5][i], acc[nb][6][i], acc[nb][7][i]};
-      *(f32x4*)(part + h * kD + dim0) = lo;
-      *(f32x4*)(part + h * kD + dim0 + 4) = hi;
+      *(f32x4*)(part + h * kD + dim0) = lo * v_scale;
+      *(f32x4*)(part + h * kD + dim0 + 4) = hi * v_scale;
     }
     if (g == 0) {
       part[kHB * kD + h] = m[nb];
@@ -257,7 +258,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads, true);
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
   if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
 }
 

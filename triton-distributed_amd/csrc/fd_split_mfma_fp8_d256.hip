@@ -11,8 +11,8 @@
 //   * V: the lane's 8 tokens x 16 dims are converted and transposed with v_perm_b32, 8 dims at
 //     a time, into the A operands of O^T[dim][head] += V^T . P^T; 16 accumulator blocks,
 //     block j holding dims 16 (4g + i) + j.
-// The per-KV-head K scale is folded into the softmax scale, the V scale multiplies the
-// finished partial once.
+// The per-KV-head K scale is folded into the softmax scale, the V scale multiplies a wave's
+// finished accumulators once.
 #include <type_traits>
 
 #include "fd_common.h"
@@ -66,6 +66,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
   char* kb = smem + wave * kWaveLds;
 
   const float kq_scale = a.sm_scale * a.k_scale[w.kvh];  // K dequantisation folded into the softmax scale
+  const float v_scale = a.v_scale[w.kvh];                // V dequantisation: once, on the finished accumulators
   const float scale2 = kq_scale * FD_LOG2E;
   const float inv_cap = SOFTCAP ? 1.0f / a.soft_cap : 0.f;
 
@@ -213,7 +214,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
 #pragma unroll
     for (int j4 = 0; j4 < 4; ++j4) {
       f32x4 o = {acc[4 * j4][i], acc[4 * j4 + 1][i], acc[4 * j4 + 2][i], acc[4 * j4 + 3][i]};
-      *(f32x4*)(part + c * kD + 16 * (4 * g + i) + 4 * j4) = o;
+      *(f32x4*)(part + c * kD + 16 * (4 * g + i) + 4 * j4) = o * v_scale;
     }
   }
   if (g == 0) {
@@ -222,7 +223,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads, true);
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
   if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);
 }
 

@@ -3,7 +3,7 @@
 // New functionality relative to the reference (python/triton_dist/kernels/nvidia/flash_decode.py:130-239 knows
 // no scaled fp8 cache); the arithmetic is that of the head_dim-128 fp8 kernel (fd_split_mfma_fp8.hip): K and V
 // bytes are dequantised exactly in registers, the K scale is folded into the softmax scale and the V scale is
-// applied once to the finished partial.
+// applied once to a wave's finished accumulators.
 //
 // A token row of one KV head is only 64 bytes -- half a cache line, and too short to fetch K or V in the MFMA
 // operand layout with wide loads -- so both go through LDS, and where the layout allows it a wave serves KH = 2
@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
   const bool head_ok = head_in_group < group;
 
   u32x4 qop[KH][2];  // Q as the MFMA B operand: lane (g, c) holds Q[head c of KV head h2][32*ks + 8g .. +7]
-  float kq_scale[KH], scale2[KH];
+  float kq_scale[KH], scale2[KH], v_scale[KH];
 #pragma unroll
   for (int h2 = 0; h2 < KH; ++h2) {
     const int kvh = KH * w.kvh + h2;
@@ -81,6 +81,7 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
     }
     kq_scale[h2] = a.sm_scale * a.k_scale[kvh];  // K dequantisation folded into the softmax scale
     scale2[h2] = kq_scale[h2] * FD_LOG2E;
+    v_scale[h2] = a.v_scale[kvh];                // V dequantisation: once, on the finished accumulators
   }
 
   const int32_t* bt_row = a.bt + (int64_t)w.b * a.sbt;
@@ -219,7 +220,7 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
   }
 
   // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge.  KH == 2: the heads of the two
-  // KV heads are stored back to back (slot h2 * group + c) as the heads of the pair, already times their V scale.
+  // KV heads are stored back to back (slot h2 * group + c) as the heads of the pair.
   wave_lds_fence();
   float* part = (float*)kb;
 #pragma unroll
@@ -229,11 +230,10 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
     lsum += __shfl_xor(lsum, 32);
     if (KH == 2 && !head_ok) continue;   // (after the shuffles: every lane takes part in them)
     const int h = KH == 2 ? h2 * group + c : c;
-    const float vs = KH == 2 ? a.v_scale[KH * w.kvh + h2] : 1.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       f32x4 o = {acc[h2][0][i], acc[h2][1][i], acc[h2][2][i], acc[h2][3][i]};
-      *(f32x4*)(part + h * kD + 4 * (4 * g + i)) = o * vs;
+      *(f32x4*)(part + h * kD + 4 * (4 * g + i)) = o * v_scale[h2];
     }
     if (g == 0) {
       part[kHB * kD + h] = m[h2];
@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
   }
   __syncthreads();
   const int nheads = KH == 2 ? a.G : min(16, a.G - w.hb * 16);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads, KH == 1);
+  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
   if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
 }
 

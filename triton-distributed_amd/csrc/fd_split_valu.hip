@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 
   // q[h][c*E .. c*E+E) in fp32, pre-multiplied by the softmax scale (and the K dequant scale).
   float kq_scale = a.sm_scale;
-  if (KV == FD_FP8_E4M3) kq_scale *= a.k_scale[w.kvh];   // the V scale multiplies the finished partial
+  if (KV == FD_FP8_E4M3) kq_scale *= a.k_scale[w.kvh];   // the V scale multiplies the finished accumulators
   const bool softcap = a.soft_cap > 0.f;
   const float inv_cap = softcap ? 1.0f / a.soft_cap : 0.f;
   const float post = softcap ? 1.0f : FD_LOG2E;  // without soft-cap scores go straight to base 2
@@ -231,10 +231,11 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   }
   float* part = (float*)smem + wave * PART;
   if (rg == 0) {
+    const float v_scale = KV == FD_FP8_E4M3 ? a.v_scale[w.kvh] : 1.0f;   // V dequantisation, once
 #pragma unroll
     for (int h = 0; h < GH; ++h) {
 #pragma unroll
-      for (int e = 0; e < E; ++e) part[h * D + c * E + e] = acc[h][e];
+      for (int e = 0; e < E; ++e) part[h * D + c * E + e] = acc[h][e] * v_scale;
       if (c == 0) {
         part[GH * D + h] = m[h];
         part[GH * D + GH + h] = l[h];
@@ -242,7 +243,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
     }
   }
   __syncthreads();
-  cta_merge_store<GH, D>(a, (const float*)smem, PART, w, nheads, KV == FD_FP8_E4M3);
+  cta_merge_store<GH, D>(a, (const float*)smem, PART, w, nheads);
   if (a.tickets) fused_combine<D>(a, w, head0, nheads, (float*)smem);  // hpw == 1 when fused
 }
 
