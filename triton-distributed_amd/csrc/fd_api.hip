@@ -52,8 +52,8 @@ bool mfma_shape_ok(int head_dim, int kv_dtype) {
 }
 
 // Tuning overrides for experiments, read once per process: FD_WAVES_PER_BLOCK (1, 2, 4 or 8 waves per (KV head,
-// split) where the caller leaves the choice to the library), FD_HEADS_PER_BLOCK (members per workgroup) and
-// FD_HEAD_BLOCK (16 or 32 query heads per wave in the head_dim-128 kernels).
+// split) where the caller leaves the choice to the library), FD_HEADS_PER_BLOCK (members per workgroup),
+// FD_HEAD_BLOCK (16 or 32 query heads per wave in the head_dim-128 kernels) and FD_NO_CHUNK.
 int env_int(const char* name) {
   const char* e = getenv(name);
   return e ? atoi(e) : 0;
@@ -102,6 +102,8 @@ constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
+constexpr int64_t kStoreThroughBytes = 16 << 20;   // partials of a step from which on they are written through
+constexpr int kMaxSplitsPerWave = 2;   // chunked work items: splits one wave walks (all but the last parked in LDS)
 
 int env_waves() {
   static const int v = env_int("FD_WAVES_PER_BLOCK");
@@ -110,6 +112,11 @@ int env_waves() {
 int env_heads() {
   static const int v = env_int("FD_HEADS_PER_BLOCK");
   return v;
+}
+// FD_NO_CHUNK=1 (experiments): one workgroup per split even where a workgroup could walk several.
+bool env_no_chunk() {
+  static const int v = env_int("FD_NO_CHUNK");
+  return v != 0;
 }
 
 // Waves per (KV head, split) when the caller does not choose: the smallest power of two that reaches
@@ -226,8 +233,18 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   a.adapt = p->split_adapt;
   a.max_pages = p->max_pages_per_seq; a.num_pages = p->num_pages;
   a.q_dtype = p->q_dtype; a.mid_dtype = p->mid_dtype;
-  a.vec_out = (p->mid_dtype == FD_F32 && aligned16(out_split) && stride_o_bs % 4 == 0 && stride_o_h % 4 == 0 &&
-               stride_o_split % 4 == 0) ? 1 : 0;
+  // rows that start on a multiple of four elements are stored four values at a time
+  a.vec_out = ((reinterpret_cast<uintptr_t>(out_split) & (4u * msz - 1)) == 0 && stride_o_bs % 4 == 0 &&
+               stride_o_h % 4 == 0 && stride_o_split % 4 == 0) ? 1 : 0;
+
+  // Tens of MB of partials left dirty in the L2s are written back when the kernel ends, with nothing to overlap;
+  // written through they leave while other workgroups stream (config 5's shape, 64 splits, 67 MB of fp32 partials:
+  // 204 -> 192 us; 4 MB of partials: no gain, so the plain store stays for those).
+  {
+    static const int forced = env_int("FD_STORE_THROUGH");   // tuning override for experiments: 1 always, 2 never
+    const int64_t partial_bytes = (int64_t)batch * p->q_heads * p->num_splits * D * msz;
+    a.store_through = a.vec_out && forced != 2 && (forced == 1 || partial_bytes >= kStoreThroughBytes) ? 1 : 0;
+  }
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
   const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
@@ -263,9 +280,26 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   }
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
+  const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
+  // Chunked work items: the caller's split count and ranges are kept exactly (they are observable in out_split), but a
+  // workgroup walks `chunk` consecutive splits, so that the chip sees as many work items as the library's own plan
+  // would launch: every work item pays the prologue (arguments -> length -> block table -> first rows) once, not once
+  // per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.
+  a.chunk = 1;
+  int chunk_wish = 1;
+  if (use_mfma && D == 128 && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
+      !env_no_chunk()) {
+    fd_params plan = *p;
+    plan.split_adapt = 0;
+    const int s_plan = fd_plan_splits(&plan, batch);
+    if (s_plan > 0 && s_plan < a.S) chunk_wish = (a.S + s_plan - 1) / s_plan;
+  }
+  a.chunk = chunk_wish;
+  const int items = (a.S + a.chunk - 1) / a.chunk;   // work items per (sequence, KV head, head block)
+  max_tok_split *= a.chunk;
   // Ranges that are certain to be busy per sequence: all of them, or, when the ranges follow each sequence's own
   // length, only the ones every sequence gets (the rest of the grid may be empty ranges).
-  const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : a.S;
+  const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : items;
   const int64_t wgs = (int64_t)batch * busy_splits * a.Hkv * a.nhb;
   // the two-block MFMA kernel needs the register file of a whole SIMD per wave: workgroups of at most 4 waves
   const int max_waves = use_mfma && (a.hbsz > 16 || pair) ? 4 : 8;
@@ -274,9 +308,19 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   const int64_t wave_target = use_mfma && !(kv_fp8 && D == 64 && !pair) ? kTargetWaves : kTargetWavesValu;
   int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
                                  : choose_waves(wgs, max_tok_split, tile, wave_target, max_waves);
+  if (a.chunk > 1) {
+    // The waves of a head take whole splits, kMaxSplitsPerWave at most: a wave keeps the finished partials of all but
+    // its last split in LDS until it has issued its last load (stores and loads of a wave retire in order, so a store
+    // between two tiles would hold back the loads behind it).
+    while (waves > 1 && waves > a.chunk) waves >>= 1;
+    int per_wave = (a.chunk + waves - 1) / waves;
+    if (per_wave > kMaxSplitsPerWave) per_wave = kMaxSplitsPerWave;
+    a.chunk = waves * per_wave;
+    a.park = per_wave - 1;
+    if (a.chunk == 1) a.park = 0;
+  }
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
-  const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
   if (use_mfma && !fuse && a.nhb > 1) {
     // more query heads per KV head than one wave serves: the head blocks of a KV head share a workgroup (largest divisor of
     // nhb that keeps the workgroup at 8 waves and the grid at one workgroup per CU), so that they read their
@@ -505,8 +549,9 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   a.s_mb = stride_mid_ob; a.s_mh = stride_mid_oh; a.s_ms = stride_mid_os; a.s_ob = stride_obs; a.s_oh = stride_oh;
   a.batch = batch; a.Hq = q_heads; a.D = p->head_dim; a.num_partials = num_partials; a.num_extra = num_extra;
   a.mode = mode; a.mid_dtype = p->mid_dtype; a.out_dtype = p->out_dtype;
-  a.vec_mid = (p->mid_dtype == FD_F32 && aligned16(mid_o) && stride_mid_ob % 4 == 0 && stride_mid_oh % 4 == 0 &&
-               stride_mid_os % 4 == 0) ? 1 : 0;
+  // rows that start on a multiple of four elements are read four values at a time
+  a.vec_mid = ((reinterpret_cast<uintptr_t>(mid_o) & (4u * dtype_size(p->mid_dtype) - 1)) == 0 && stride_mid_ob % 4 == 0 &&
+               stride_mid_oh % 4 == 0 && stride_mid_os % 4 == 0) ? 1 : 0;
   a.all_slots_written = all_slots_written ? 1 : 0;
   if (p->split_align < 0 || p->split_align > 4096 || (p->split_align & (p->split_align - 1)))
     return fail(FD_ERR_INVALID_ARG, "fd_combine: split_align %d (0 or a power of two <= 4096)", p->split_align);

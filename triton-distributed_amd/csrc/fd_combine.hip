@@ -73,13 +73,23 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
 
   const int r = tid >> a.cg_shift;
   const int c = col0 / 4 + (tid - (r << a.cg_shift));   // 128-bit column group within the row
-  const bool vec_mid = a.mid_dtype == FD_F32 && a.vec_mid;
+  const bool vec_mid = a.vec_mid != 0;
   auto load_row = [&](int s) -> f32x4 {   // this thread's 4 columns of partial s
     f32x4 o;
     if (s < S) {
       const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
-      if (vec_mid) {
+      if (vec_mid && a.mid_dtype == FD_F32) {
         o = *(const f32x4*)((const float*)a.mid_o + off);
+      } else if (vec_mid) {   // four packed 16-bit values in one 64-bit load
+        const u32x2 w = *(const u32x2*)((const uint16_t*)a.mid_o + off);
+        if (a.mid_dtype == FD_F16) {
+          // halves taken apart as integers: with 2-element half vectors the compiler used the first dword twice
+          o = f32x4{f16_bits_to_f32(w[0] & 0xffffu), f16_bits_to_f32(w[0] >> 16), f16_bits_to_f32(w[1] & 0xffffu),
+                    f16_bits_to_f32(w[1] >> 16)};
+        } else {
+          o = f32x4{bf16_bits_to_f32(w[0] & 0xffffu), bf16_bits_to_f32(w[0] >> 16), bf16_bits_to_f32(w[1] & 0xffffu),
+                    bf16_bits_to_f32(w[1] >> 16)};
+        }
       } else {
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = load_as_f32(a.mid_o, off + k, a.mid_dtype);
@@ -156,65 +166,89 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   }
 }
 
-// Few partials (<= kSmallMax), fp32 and 128-bit aligned, produced by this library's split kernel in the
-// same call: every slot is written (an empty split holds out = 0, lse = -inf), so validity needs no
-// kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which leaves one
-// dependent memory round trip.  Thread (r, c): partial r (and r + ROWS), 128-bit column chunk c.
-constexpr int kSmallMax = kCombineSmallMax;
-
-template <int D>
-__global__ void __launch_bounds__(kCombineThreads) fd_combine_small_kernel(const CombineArgs a) {
+// Up to MAXP (16 or 32) partials produced by this library's split kernel in the same call, rows readable four values at a time,
+// LSEs in their own fp32 buffer: every slot is written (an empty split holds out = 0, lse = -inf), so validity needs
+// no kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which leaves one dependent
+// memory round trip.  The kernel is short on purpose: one workgroup per output row on a chip that the step's split
+// kernel has just vacated runs at one wave per SIMD, where every instruction of the wave is latency.  Thread (r, c):
+// partials r, r + ROWS, ... and 128-bit column chunk c.  Every thread reads all LSEs of the row itself (the same few
+// cache lines for the whole workgroup) for the maximum, so nothing goes through LDS before the final sum.
+template <int D, int MAXP>
+__global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const CombineArgs a) {
   constexpr int CG = D / 4;
   constexpr int ROWS = kCombineThreads / CG;
+  constexpr int PASSES = (MAXP + ROWS - 1) / ROWS;
   __shared__ __align__(16) float s_acc[ROWS][D];
+  __shared__ float s_l[ROWS];
   const int tid = threadIdx.x;
   const int b = blockIdx.x / a.Hq;
   const int h = blockIdx.x - b * a.Hq;
   const int S = a.num_partials;
-  const float* mid = (const float*)a.mid_o + (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
+  const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
+  const float* lse_row = a.mid_lse + ((int64_t)b * a.Hq + h) * S;
   const int r = tid / CG;
   const int c = tid - r * CG;
-  constexpr int PASSES = (kSmallMax + ROWS - 1) / ROWS;
   f32x4 o[PASSES];
+  float own[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int s = r + p * ROWS;
-    o[p] = s < S ? *(const f32x4*)(mid + (int64_t)s * a.s_ms + 4 * c) : f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  float lse[kSmallMax];
-#pragma unroll
-  for (int s = 0; s < kSmallMax; ++s) {
-    lse[s] = -INFINITY;
-    if (s < S) lse[s] = a.mid_lse ? a.mid_lse[((int64_t)b * a.Hq + h) * S + s] : mid[(int64_t)s * a.s_ms + D];
+    o[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+    own[p] = -INFINITY;
+    if (s < S) {
+      const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
+      if (a.mid_dtype == FD_F32) {
+        o[p] = *(const f32x4*)((const float*)a.mid_o + off);
+      } else {
+        const u32x2 w = *(const u32x2*)((const uint16_t*)a.mid_o + off);
+        if (a.mid_dtype == FD_F16) {
+          o[p] = f32x4{f16_bits_to_f32(w[0] & 0xffffu), f16_bits_to_f32(w[0] >> 16), f16_bits_to_f32(w[1] & 0xffffu),
+                       f16_bits_to_f32(w[1] >> 16)};
+        } else {
+          o[p] = f32x4{bf16_bits_to_f32(w[0] & 0xffffu), bf16_bits_to_f32(w[0] >> 16), bf16_bits_to_f32(w[1] & 0xffffu),
+                       bf16_bits_to_f32(w[1] >> 16)};
+        }
+      }
+      own[p] = lse_row[s];
+    }
   }
   float M = -INFINITY;
+  if ((S & 3) == 0) {   // the row of LSEs is 16-byte aligned
 #pragma unroll
-  for (int s = 0; s < kSmallMax; ++s) M = fmaxf(M, lse[s]);
+    for (int q = 0; q < MAXP / 4; ++q) {
+      if (4 * q < S) {
+        const f32x4 v = *(const f32x4*)(lse_row + 4 * q);
+        M = fmaxf(fmaxf(M, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
+      }
+    }
+  } else {
+    for (int q = 0; q < S; ++q) M = fmaxf(M, lse_row[q]);
+  }
   float L = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   if (M > -INFINITY) {
 #pragma unroll
-    for (int s = 0; s < kSmallMax; ++s) L += __expf(lse[s] - M);   // exp(-inf) = 0 for empty / absent splits
-#pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      const int s = r + p * ROWS;
-      float wgt = 0.f;
-#pragma unroll
-      for (int q = 0; q < kSmallMax; ++q) wgt = q == s ? __expf(lse[q] - M) : wgt;
+      const float wgt = __expf(own[p] - M);   // exp(-inf) = 0 for empty / absent splits
       acc += o[p] * wgt;
+      L += wgt;
     }
   }
   *(f32x4*)&s_acc[r][4 * c] = acc;
+  if (c == 0) s_l[r] = L;
   __syncthreads();
   if (tid < D) {
-    float v = 0.f;
+    float v = 0.f, Lsum = 0.f;
 #pragma unroll
-    for (int i = 0; i < ROWS; ++i) v += s_acc[i][tid];
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int i = 0; i < ROWS; ++i) {
+      v += s_acc[i][tid];
+      Lsum += s_l[i];
+    }
+    const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
     const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
     store_from_f32(a.out, out_base + tid, a.out_dtype, v * inv);
     if (tid == 0) {
-      const float res = L > 0.f ? M + __logf(L) : -INFINITY;
+      const float res = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
       if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, res);
       if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = res;
     }
@@ -267,8 +301,12 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   CombineArgs a = args;
   const int64_t rows = (int64_t)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
-  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 &&
-                     a.num_partials <= kSmallMax && a.mid_dtype == FD_F32 && a.vec_mid;
+  // the short kernel: this library's own partials in the same call, all slots written, at most 32 of them (with 64 a
+  // thread would hold 8 rows and 64 LSEs, and the registers for that cost the occupancy that large batches need:
+  // config 5's shape with 64 splits 24.7 us against 13 us in the general kernel)
+  const int np_own = a.num_partials <= 16 ? 16 : 32;
+  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 && a.num_partials <= 32 &&
+                     a.vec_mid && a.mid_lse && (reinterpret_cast<uintptr_t>(a.mid_lse) & 15u) == 0;
   // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
   // one workgroup per CU and a thread would still have more than two partials to walk.
   int cg = a.D / 4;
@@ -279,12 +317,14 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   const int64_t wgs = small ? rows : rows * (a.D / 4 / cg);
   if (wgs >= ((int64_t)1 << 31)) return FD_ERR_TOO_LARGE;
   const unsigned grid = (unsigned)wgs;
+#define FD_OWN(D_) (np_own == 16 ? fd_combine_own_kernel<D_, 16> : fd_combine_own_kernel<D_, 32>)
   switch (a.D) {
-    case 64: kern = small ? fd_combine_small_kernel<64> : fd_combine_kernel<64>; break;
-    case 128: kern = small ? fd_combine_small_kernel<128> : fd_combine_kernel<128>; break;
-    case 256: kern = small ? fd_combine_small_kernel<256> : fd_combine_kernel<256>; break;
+    case 64: kern = small ? FD_OWN(64) : fd_combine_kernel<64>; break;
+    case 128: kern = small ? FD_OWN(128) : fd_combine_kernel<128>; break;
+    case 256: kern = small ? FD_OWN(256) : fd_combine_kernel<256>; break;
     default: return FD_ERR_UNSUPPORTED;
   }
+#undef FD_OWN
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }

@@ -50,12 +50,20 @@ struct SplitArgs {
                       // heads than a wave serves: the blocks read the same K/V rows in step, so the rows come
                       // from HBM once)
   int32_t grid_x;   // workgroups per (sequence, split)
-  int32_t vec_out;  // 1: every out row start is 16-byte aligned (128-bit stores allowed)
+  int32_t vec_out;  // 1: every out row starts on a multiple of four elements (one 128-bit store per four fp32 values, one
+                    // 64-bit store per four 16-bit values)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
   int32_t per_mask;               // split_align - 1 (0: the reference's ranges): tokens per split are rounded up
   int32_t adapt;                  // fd_params.split_adapt: ranges per sequence by its own length (0: always S)
   int32_t skip_empty;             // 1: a workgroup whose range is empty writes nothing (the combine knows the ranges)
+  int32_t chunk;                  // consecutive splits one workgroup walks (1: one split per workgroup).  Above 1 every
+                                  // wave owns whole splits -- ceil(chunk / nsub) consecutive ones -- and stores one
+                                  // partial per split itself, so the caller sees exactly S partials in the reference
+                                  // layout while the chip sees S / chunk long work items
+  int32_t store_through;          // 1: partials are written through to memory (sc0 sc1) instead of being left dirty in
+                                  // the XCD's L2 until the kernel ends; pays off for tens of MB of partials
+  int32_t park;                   // chunked work items: finished partials a wave parks in LDS besides its last one
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
   int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
@@ -77,7 +85,8 @@ struct CombineArgs {
   const float* extra_lse;
   int64_t s_mb, s_mh, s_ms, s_ob, s_oh;
   int32_t batch, Hq, D, num_partials, num_extra, mode, mid_dtype, out_dtype;
-  int32_t vec_mid;  // 1: every mid_o row start is 16-byte aligned (128-bit loads allowed)
+  int32_t vec_mid;  // 1: every mid_o row starts on a multiple of four elements (128-bit loads of fp32, 64-bit loads of
+                    // 16-bit partials)
   int32_t cg_shift; // log2 of the 128-bit column groups a workgroup of the general kernel covers (set by the launcher)
   int32_t per_mask;           // as SplitArgs::per_mask, for the validity of split ranges
   int32_t adapt;              // as SplitArgs::adapt
@@ -125,6 +134,9 @@ struct AppendArgs {
 // ---------------------------------------------------------------- scalar conversions
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t lo16) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)lo16);
+}
 
 __device__ __forceinline__ float load_as_f32(const void* p, int64_t idx, int dtype) {
   switch (dtype) {
@@ -172,6 +184,37 @@ __device__ __forceinline__ float fd_softcap(float x, float cap, float inv_cap) {
 __device__ __forceinline__ u32x4 load_stream_b128(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
 __device__ __forceinline__ u32x2 load_stream_b64(const void* p) { return __builtin_nontemporal_load((const u32x2*)p); }
 
+// Four consecutive values of a partial row that starts on a multiple of four elements (SplitArgs::vec_out): one
+// 128-bit store for fp32, one 64-bit store of four packed values for fp16 / bf16.  through: written through to memory
+// (sc0 sc1).  The write-through form is inline assembly, which the compiler does not count in vmcnt: only for stores
+// that no vector-memory load of the same wave follows.
+__device__ __forceinline__ void store_partial4(void* base, int64_t off, int dtype, f32x4 o, bool through) {
+  if (dtype == FD_F32) {
+    float* p = (float*)base + off;
+    if (through) {
+      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(o) : "memory");
+    } else {
+      *(f32x4*)p = o;
+    }
+  } else {
+    const f32x2 lo = {o[0], o[1]}, hi = {o[2], o[3]};
+    u32x2 w;
+    if (dtype == FD_F16) {
+      w[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, f16x2));
+      w[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, f16x2));
+    } else {
+      w[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+      w[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+    }
+    uint16_t* p = (uint16_t*)base + off;
+    if (through) {
+      asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+    } else {
+      *(u32x2*)p = w;
+    }
+  }
+}
+
 // Orders LDS accesses of one wave: lanes of a wave exchange data through LDS
 // without a workgroup barrier (the LDS queue of a wave is in order); this only
 // stops the compiler from moving accesses across the point.
@@ -192,10 +235,10 @@ __device__ __forceinline__ void fd_fetch_args_now(const SplitArgs& a) {
   FD_PIN(sq_b); FD_PIN(sq_h); FD_PIN(sk_t); FD_PIN(sk_h); FD_PIN(sv_t); FD_PIN(sv_h); FD_PIN(sbt);
   FD_PIN(sm_scale); FD_PIN(batch); FD_PIN(G); FD_PIN(S); FD_PIN(P); FD_PIN(max_pages); FD_PIN(num_pages);
   FD_PIN(div_magic); FD_PIN(div_shift); FD_PIN(nhb); FD_PIN(hpw); FD_PIN(nsub); FD_PIN(member_hb); FD_PIN(s_magic);
-  FD_PIN(s_shift); FD_PIN(per_mask); FD_PIN(adapt); FD_PIN(skip_empty); FD_PIN(order_items);
+  FD_PIN(s_shift); FD_PIN(per_mask); FD_PIN(adapt); FD_PIN(skip_empty); FD_PIN(order_items); FD_PIN(chunk);
   // what the epilogue reads, so that it does not wait for the argument segment either
   FD_PIN(out); FD_PIN(lse); FD_PIN(so_b); FD_PIN(so_h); FD_PIN(so_s); FD_PIN(tickets); FD_PIN(mid_dtype);
-  FD_PIN(vec_out); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
+  FD_PIN(vec_out); FD_PIN(store_through); FD_PIN(park); FD_PIN(no_lse); FD_PIN(out_dtype); FD_PIN(num_extra); FD_PIN(lse_column);
 #undef FD_PIN
 }
 
@@ -252,6 +295,9 @@ struct WorkItem {
   int hb0;    // first head block of the workgroup
   int sub;    // token sub-range index of this wave
   int nsub;   // token sub-ranges (waves per head)
+  // chunked work items (SplitArgs::chunk > 1): this wave owns the splits s .. s + ns - 1 (ns may be 0) of per tokens
+  // each, i.e. the tokens [start, end)
+  int ns, per;
 };
 
 __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
@@ -312,11 +358,26 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     }
     w.nsub = a.nsub;
   }
-  w.s = min(s, a.S - 1);
   int64_t cap = (int64_t)a.max_pages * a.P;
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
   const int per = tokens_per_range(kv_len, a.S, a.s_magic, a.s_shift, a.per_mask, a.adapt);
+  w.per = per;
+  if (a.chunk > 1) {
+    // s counts work items of a.chunk splits; the waves of a head share them out in runs of whole splits
+    const int ns = (a.chunk + w.nsub - 1) / w.nsub;
+    const int first = s * a.chunk + w.sub * ns;
+    const int lim = min(min((s + 1) * a.chunk, a.S), first + ns);
+    w.s = first;
+    w.ns = max(lim - first, 0);
+    const int64_t st = (int64_t)per * first, en = (int64_t)per * (first + w.ns);
+    w.start = st > kv_len ? kv_len : (int)st;
+    w.end = en > kv_len ? kv_len : (int)en;
+    w.skip = false;
+    return w;
+  }
+  w.s = min(s, a.S - 1);
+  w.ns = 1;
   int64_t st = (int64_t)per * w.s;
   w.start = st > kv_len ? kv_len : (int)st;
   int64_t en = st + per;
@@ -407,8 +468,8 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
       for (int i = 0; i < 4; ++i) store_f32_agent((float*)a.out + off + i, o[i]);
       if (d == 0) store_f32_agent(a.lse ? a.lse + ((int64_t)w.b * a.Hq + head) * a.S + w.s : (float*)a.out + off + D, lse);
     } else {
-      if (a.mid_dtype == FD_F32 && a.vec_out) {
-        *(f32x4*)((float*)a.out + off) = o;
+      if (a.vec_out) {
+        store_partial4(a.out, off, a.mid_dtype, o, a.store_through != 0);
       } else {
         for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
       }
@@ -423,9 +484,52 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
   }
 }
 
+// Chunked work items: ONE wave stores the finished partial of split s for its own HB head slots, from an LDS buffer
+// `part` of its own (same layout as one wave's slice in cta_merge_store; the wave has ordered its LDS writes before
+// the call).  Called at the end of the wave's run only: on this target stores and loads of a wave retire in order
+// (one vmcnt), so a store issued between two tiles would hold back every later K/V load until it is acknowledged.  Rows are read back row-major, so a store instruction covers whole 512-byte rows.  empty: the split holds no
+// token (out = 0, lse = -inf; `part` is not read).
+template <int HB, int D>
+__device__ __forceinline__ void wave_store_partial(const SplitArgs& a, const float* part, int b, int head0, int nheads,
+                                                   int s, bool empty) {
+  const int lane = threadIdx.x & 63;
+  constexpr int D4 = D / 4;          // lanes per row
+  constexpr int RPI = 64 / D4;       // rows per store instruction
+  static_assert(D4 <= 64 && HB % RPI == 0, "one wave covers whole rows");
+  const int d = (lane % D4) * 4;
+#pragma unroll
+  for (int r = 0; r < HB / RPI; ++r) {
+    const int h = r * RPI + lane / D4;
+    if (h >= nheads) continue;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    float lse = -INFINITY;
+    if (!empty) {
+      const float M = part[HB * D + h];
+      const float L = part[HB * D + HB + h];
+      const float inv = L > 0.f ? 1.0f / L : 0.f;
+      o = *(const f32x4*)(part + h * D + d) * inv;
+      lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+    }
+    const int head = head0 + h;
+    const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
+    if (a.vec_out) {
+      store_partial4(a.out, off, a.mid_dtype, o, a.store_through != 0);
+    } else {
+      for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
+    }
+    if (d == 0 && !a.no_lse) {
+      if (a.lse) {
+        a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
+      } else {
+        store_from_f32(a.out, off + D, a.mid_dtype, lse);
+      }
+    }
+  }
+}
+
 // Fused combine: called by every thread of the workgroup after cta_merge_store() (which, in this
-// mode, wrote the fp32 partials with agent-scope stores).  Every thread waits for its stores to
-// complete, one thread takes a ticket for the (sequence, KV head, head block) group, and the
+// mode, wrote the fp32 partials with agent-scope stores).  Every wave waits for its stores to
+// be acknowledged (an explicit vmcnt(0) wait), one thread takes a ticket for the (sequence, KV head, head block) group, and the
 // workgroup that draws the last ticket merges the group's S partials (and the extra ones) into the
 // final output with the stand-alone combine kernel's weights softmax(LSE)_s.  No workgroup ever
 // waits for another one.  s_lse: LDS scratch of at least (S + num_extra) * nheads floats.
@@ -435,7 +539,15 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
   __shared__ int s_last;
   const int tid = threadIdx.x;
   const int nth = 64 * a.hpw * a.nsub;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // vmcnt(0): the write-through stores have completed
+  // Every wave waits here until all its partial stores have been acknowledged: they are agent-scope write-through
+  // stores, so an acknowledged store has left this XCD's L2 and is what an agent-scope load from any XCD returns.  A
+  // workgroup-scope release fence would not do: outside threadgroup-split mode it orders LDS traffic only (waves of a
+  // workgroup share their CU's vector cache) and leaves vector-memory stores in flight.  The barrier then collects
+  // "all stores of all waves acknowledged", and only after it does thread 0 take the ticket, itself an agent-scope
+  // read-modify-write performed at the same memory-side point the stores went to.  The workgroup that draws the last
+  // ticket therefore takes it after every other workgroup's partials have landed, and its agent-scope loads (which
+  // do not hit in its own L2) are issued after the ticket has returned (s_last goes through LDS and a barrier).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (tid == 0) {
     int32_t* t = a.tickets + ((int64_t)w.b * a.Hkv + w.kvh) * a.nhb + w.hb;
@@ -611,7 +723,8 @@ __device__ __forceinline__ void fd_schedule_items_block(int tid, int batch, LenF
 // Launch grid of the split kernels (see decode_work_item).
 inline dim3 fd_split_grid(const SplitArgs& a) {
   if (a.adapt > 0 && !a.order_items) return dim3((unsigned)a.grid_x, (unsigned)a.batch, (unsigned)a.S);
-  return dim3((unsigned)a.grid_x, (unsigned)a.S, (unsigned)a.batch);
+  const int items = a.chunk > 1 ? (a.S + a.chunk - 1) / a.chunk : a.S;   // work items per sequence
+  return dim3((unsigned)a.grid_x, (unsigned)items, (unsigned)a.batch);
 }
 
 // Launchers implemented in the kernel translation units (host side).

@@ -49,7 +49,12 @@ static_assert(wave_lds(1) >= (16 * kD + 2 * 16) * 4 && wave_lds(2) >= kKTile, "p
 #define FD_MFMA_OCC
 #endif
 
-template <typename T, bool SOFTCAP, int NB>
+// CHUNK: a workgroup walks SplitArgs::chunk consecutive splits.  Every wave owns whole splits: it streams their tiles
+// as one run -- Q operands, table row and the K/V pipeline stay alive across a split boundary -- puts each finished
+// split's state aside in LDS, and at the end normalises and stores one partial per split itself (no workgroup merge),
+// so the caller gets exactly S partials in the reference layout [B, Hq, S, D(+1)] (flash_decode.py:193-195, 235-239)
+// from S / chunk long work items.
+template <typename T, bool SOFTCAP, int NB, bool CHUNK>
 __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma16_kernel(const SplitArgs a) {
   constexpr int kHB = 16 * NB;             // head slots per wave
   constexpr int kWaveLds = wave_lds(NB);
@@ -62,6 +67,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
 
   const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
   if (w.skip) return;   // empty range, and the combine does not expect a partial from it
+  if (CHUNK && w.ns <= 0) return;   // more waves than splits in the last work item of a sequence (no barrier follows)
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
   const int tpw = (ntiles + w.nsub - 1) / w.nsub;
@@ -95,6 +101,13 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
 
   // lane (l & 31) looks up token start + 32t + (l & 31)
   auto tile_slot = [&](int t, int& slot) -> int { return fd_tile_slot<kTile>(a, w, bt_row, t, lane & 31, slot); };
+  // ... or, with chunked work items, token n0 + (l & 31) of the tile that starts at n0 in a split that ends at n_end
+  auto token_slot = [&](int n0, int n_end, int& slot) -> int {
+    const int n = min(n0 + (lane & 31), n_end - 1);
+    const int pidx = page_index(a, n);
+    slot = n - pidx * a.P;
+    return bt_row[pidx];
+  };
 
   u32x4 kraw[8], vraw[8];
   int rows[8];
@@ -129,7 +142,9 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
   // One tile.  HAS_NEXT is a compile-time flag (the last tile of the wave is peeled off the loop),
   // so the steady-state loop has no branch around a load and the wait counts stay exact:
   // K(t+1) and V(t+1) are in flight while tile t is being computed.
-  auto tile = [&](int t, auto has_next_tag) {
+  // n0 / n_end: first token of the tile and end of its split (for the mask); lookup2(slot): table entry and slot of
+  // this lane's token two tiles ahead.
+  auto tile = [&](const int n0, const int n_end, auto&& lookup2, auto has_next_tag) {
     constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
     // ---- K tile -> LDS, then start fetching the next tile's K into the freed registers
     wave_lds_fence();
@@ -145,7 +160,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       __builtin_amdgcn_sched_barrier(0);
       fetch_rows(pg_next, slot_next);
       issue_k();
-      pg_next = tile_slot(min(t + 2, t1 - 1), slot_next);
+      pg_next = lookup2(slot_next);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- S^T = K . Q^T
@@ -163,8 +178,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       }
     }
     // ---- online softmax (head 16*nb + c, tokens tau(g, 0..7))
-    const int n0 = w.start + t * kTile;
-    const bool full = n0 + kTile <= w.end;
+    const bool full = n0 + kTile <= n_end;
     u32x4 pop[NB];  // P^T as the B operand: element e <-> token tau(g, e)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -187,7 +201,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       if (!full) {   // only the last tile of a range has tokens to mask (wave-uniform branch)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-          if (n0 + 4 * g + (i & 3) + 16 * (i >> 2) >= w.end) x[i] = -INFINITY;
+          if (n0 + 4 * g + (i & 3) + 16 * (i >> 2) >= n_end) x[i] = -INFINITY;
       }
       bool moved;
       const float alpha = fd_softmax_step(x, m[nb], l[nb], moved);
@@ -229,54 +243,132 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
     }
   };
 
-  if (t0 < t1) {
-    int slot0;
-    const int pg0 = tile_slot(t0, slot0);
-    pg_next = tile_slot(min(t0 + 1, t1 - 1), slot_next);
-    // same request order as in the loop (table entry of the next tile before the K/V rows), so the
-    // wait counts at the loop head are exact on the first iteration as well
-    __builtin_amdgcn_sched_barrier(0);
-    fetch_rows(pg0, slot0);
-    issue_k();
-    issue_v();
-    __builtin_amdgcn_sched_barrier(0);
-    for (int t = t0; t < t1 - 1; ++t) tile(t, std::true_type{});
-    tile(t1 - 1, std::false_type{});
-  }
-
-  // ---- wave result -> LDS (the wave's own staging buffer), then workgroup merge
-  wave_lds_fence();
+  // A wave's finished state -> its own LDS buffer (the K staging buffer), in cta_merge_store's layout.
   float* part = (float*)kb;
+  auto stage_partial = [&](float* part) {
+    wave_lds_fence();
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    float lsum = l[nb];
-    lsum += __shfl_xor(lsum, 16);
-    lsum += __shfl_xor(lsum, 32);
-    const int h = 16 * nb + c;
+    for (int nb = 0; nb < NB; ++nb) {
+      float lsum = l[nb];
+      lsum += __shfl_xor(lsum, 16);
+      lsum += __shfl_xor(lsum, 32);
+      const int h = 16 * nb + c;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f32x4 lo = {acc[nb][0][i], acc[nb][1][i], acc[nb][2][i], acc[nb][3][i]};
-      f32x4 hi = {acc[nb][4][i], acc[nb][5][i], acc[nb][6][i], acc[nb][7][i]};
-      *(f32x4*)(part + h * kD + 32 * g + 8 * i) = lo;
-      *(f32x4*)(part + h * kD + 32 * g + 8 * i + 4) = hi;
+      for (int i = 0; i < 4; ++i) {
+        f32x4 lo = {acc[nb][0][i], acc[nb][1][i], acc[nb][2][i], acc[nb][3][i]};
+        f32x4 hi = {acc[nb][4][i], acc[nb][5][i], acc[nb][6][i], acc[nb][7][i]};
+        *(f32x4*)(part + h * kD + 32 * g + 8 * i) = lo;
+        *(f32x4*)(part + h * kD + 32 * g + 8 * i + 4) = hi;
+      }
+      if (g == 0) {
+        part[kHB * kD + h] = m[nb];
+        part[kHB * kD + kHB + h] = lsum;
+      }
     }
-    if (g == 0) {
-      part[kHB * kD + h] = m[nb];
-      part[kHB * kD + kHB + h] = lsum;
-    }
-  }
-  __syncthreads();
+  };
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
-  if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
+
+  if constexpr (CHUNK) {
+    // Wave-uniform cursors over the tiles of the wave's splits: a tile starts at `base` inside a split that ends at
+    // `end`; the tile after the last one of a split is the first one of the next split (splits are `per` tokens apart,
+    // only the last non-empty one may be shorter).  The cursor stops on the wave's last tile.
+    const int per = __builtin_amdgcn_readfirstlane(w.per);
+    const int run_end = __builtin_amdgcn_readfirstlane(w.end);
+    const int head0 = w.kvh * a.G + w.hb * kHB;
+    const int s_cur = __builtin_amdgcn_readfirstlane(w.s);
+    const int s_lim = s_cur + __builtin_amdgcn_readfirstlane(w.ns);
+    struct Cur { int base, end; };
+    auto advance = [&](const Cur cur) -> Cur {
+      Cur n = cur;
+      n.base += kTile;
+      if (n.base >= cur.end) {
+        n.base = cur.end;
+        n.end = min(cur.end + per, run_end);
+      }
+      return n.base >= run_end ? cur : n;
+    };
+    // Finished partials other than the wave's last one wait in LDS behind the staging buffers (a.park slots per
+    // wave); all of them are stored when the wave has issued its last load.
+    constexpr int kPartFloats = kHB * kD + 2 * kHB;
+    float* park = (float*)(smem + a.hpw * a.nsub * kWaveLds) + (size_t)(wave * a.park) * kPartFloats;
+    int parked = 0;
+    bool last_staged = false;
+    Cur cur{__builtin_amdgcn_readfirstlane(w.start), 0};
+    cur.end = min(cur.base + per, run_end);
+    if (cur.base < run_end) {
+      Cur look = advance(cur);
+      int slot0;
+      const int pg0 = token_slot(cur.base, cur.end, slot0);
+      pg_next = token_slot(look.base, look.end, slot_next);
+      look = advance(look);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_rows(pg0, slot0);
+      issue_k();
+      issue_v();
+      __builtin_amdgcn_sched_barrier(0);
+      auto lookup2 = [&](int& slot) -> int { return token_slot(look.base, look.end, slot); };
+      while (!(cur.end >= run_end && cur.base + kTile >= cur.end)) {   // all tiles but the wave's last one
+        tile(cur.base, cur.end, lookup2, std::true_type{});
+        if (cur.base + kTile >= cur.end) {   // that was the last tile of a split
+          stage_partial(park + parked * kPartFloats);
+          ++parked;
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            m[nb] = -INFINITY;
+            l[nb] = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[nb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+        cur = advance(cur);
+        look = advance(look);
+      }
+      tile(cur.base, cur.end, lookup2, std::false_type{});
+      stage_partial(part);
+      last_staged = true;
+    }
+    wave_lds_fence();
+    for (int i = 0; s_cur + i < s_lim; ++i) {   // splits beyond the sequence's end are stored as empty
+      const bool empty = i > parked || (i == parked && !last_staged);
+      wave_store_partial<kHB, kD>(a, i < parked ? park + i * kPartFloats : part, w.b, head0, nheads, s_cur + i, empty);
+    }
+  } else {
+    if (t0 < t1) {
+      int slot0;
+      const int pg0 = tile_slot(t0, slot0);
+      pg_next = tile_slot(min(t0 + 1, t1 - 1), slot_next);
+      // same request order as in the loop (table entry of the next tile before the K/V rows), so the
+      // wait counts at the loop head are exact on the first iteration as well
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_rows(pg0, slot0);
+      issue_k();
+      issue_v();
+      __builtin_amdgcn_sched_barrier(0);
+      for (int t = t0; t < t1 - 1; ++t)
+        tile(w.start + t * kTile, w.end, [&](int& slot) -> int { return tile_slot(min(t + 2, t1 - 1), slot); },
+             std::true_type{});
+      tile(w.start + (t1 - 1) * kTile, w.end, [&](int& slot) -> int { return tile_slot(t1 - 1, slot); },
+           std::false_type{});
+    }
+
+    // ---- wave result -> LDS, then workgroup merge
+    stage_partial(part);
+    __syncthreads();
+    cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
+    if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
+  }
 }
 
 }  // namespace
 
+template <typename T, bool CHUNK>
+static auto pick_kernel2(bool soft_cap, int nb) -> void (*)(const SplitArgs) {
+  if (nb == 2) return soft_cap ? fd_split_mfma16_kernel<T, true, 2, CHUNK> : fd_split_mfma16_kernel<T, false, 2, CHUNK>;
+  return soft_cap ? fd_split_mfma16_kernel<T, true, 1, CHUNK> : fd_split_mfma16_kernel<T, false, 1, CHUNK>;
+}
 template <typename T>
-static auto pick_kernel(bool soft_cap, int nb) -> void (*)(const SplitArgs) {
-  if (nb == 2) return soft_cap ? fd_split_mfma16_kernel<T, true, 2> : fd_split_mfma16_kernel<T, false, 2>;
-  return soft_cap ? fd_split_mfma16_kernel<T, true, 1> : fd_split_mfma16_kernel<T, false, 1>;
+static auto pick_kernel(bool soft_cap, int nb, bool chunk) -> void (*)(const SplitArgs) {
+  return chunk ? pick_kernel2<T, true>(soft_cap, nb) : pick_kernel2<T, false>(soft_cap, nb);
 }
 
 // a.hbsz = query heads per head block: up to 16 (one MFMA column block per wave) or 32 (two)
@@ -285,15 +377,16 @@ int fd_launch_split_mfma(hipStream_t stream, const SplitArgs& a, int kv_dtype, i
   const unsigned block = 64u * waves;
   const int nb = a.hbsz > 16 ? 2 : 1;
   size_t lds = (size_t)waves * wave_lds(nb);
+  if (a.chunk > 1) lds += (size_t)waves * a.park * (16 * nb * kD + 2 * 16 * nb) * 4;   // parked partials
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
     const size_t need = (size_t)(a.S + a.num_extra) * 16 * nb * 4;
     if (need > lds) lds = need;
   }
   void (*kern)(const SplitArgs) = nullptr;
   if (kv_dtype == FD_BF16) {
-    kern = pick_kernel<__bf16>(soft_cap, nb);
+    kern = pick_kernel<__bf16>(soft_cap, nb, a.chunk > 1);
   } else if (kv_dtype == FD_F16) {
-    kern = pick_kernel<_Float16>(soft_cap, nb);
+    kern = pick_kernel<_Float16>(soft_cap, nb, a.chunk > 1);
   } else {
     return FD_ERR_UNSUPPORTED;
   }

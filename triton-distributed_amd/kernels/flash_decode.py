@@ -40,7 +40,7 @@ from typing import Optional
 
 import torch
 
-from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F32, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
+from .._lib import (FD_BF16, FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F16, FD_F32, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
                     FdParams, check, fd_dtype_of, load_library, stream_handle)
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
@@ -77,6 +77,17 @@ def auto_split_bound(capacity: int) -> int:
     """Upper bound of the split count when the caller leaves it to the library (``kv_split == -1`` and no
     ``output_split``): the reference's 32 (flash_decode.py:779), more for block tables of more than 16384 tokens."""
     return max(DEFAULT_KV_SPLITS, min(MAX_AUTO_KV_SPLITS, capacity // 512))
+
+
+def internal_partial_dtype(out_dtype, plan_splits, fuse_combine):
+    """Element type of the partials when they stay inside the library (the LSEs are always fp32, in their own
+    buffer).  Planned splits are few and long: fp32.  A caller who insists on exactly ``kv_split`` splits
+    (``plan_splits=False``) gets partials in the output's precision when that is 16-bit -- what the reference's
+    intra-rank wrapper allocates (flash_decode.py:867-868; the plain one fp16 whatever the inputs, :783-784): with 32
+    or 64 splits per sequence the partials are megabytes that the split kernel writes and the combine reads back."""
+    if plan_splits or fuse_combine or out_dtype not in (torch.float16, torch.bfloat16):
+        return FD_F32
+    return FD_F16 if out_dtype == torch.float16 else FD_BF16
 
 
 def _require_cuda(*tensors):
@@ -229,7 +240,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
                 hold.record_stream(stream)
         mid_ptr = hold.data_ptr() if hold is not None else None
         lse_split_ptr = mid_ptr + 4 * n_o if hold is not None else None
-        mid_dtype = FD_F32
+        mid_dtype = internal_partial_dtype(output_combine.dtype if output_combine is not None else q.dtype,
+                                           plan_splits, fuse_combine)
         so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
     else:
         assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
