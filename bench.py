@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-targets", action="store_true",
+                    help="skip the other north-star figures (exact split counts, configs 3, 4, 5) that the default "
+                         "run measures besides the headline")
     ap.add_argument("--no-write-side", action="store_true",
                     help="skip the timing of the step before the decode (rotary + KV append)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences the CPU baseline times (0 = choose)")
@@ -72,6 +75,115 @@ def _time_us(torch, fn, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def make_pools(torch, wl, dev, n):
+    """Independent KV pools for the steps to rotate over: pool 0 holds the seeded data (the one checked against
+    the CPU baseline), the others other random bits of the same distribution."""
+    pools = [(wl.k_cache, wl.v_cache)]
+    for _ in range(1, max(1, n)):
+        if wl.k_cache.dtype in (torch.float16, torch.bfloat16, torch.float32):
+            k = torch.empty_like(wl.k_cache).normal_()
+            v = torch.empty_like(wl.v_cache).normal_()
+        else:  # fp8 bit patterns: shuffle pages of pool 0
+            perm = torch.randperm(wl.k_cache.shape[0], device=dev)
+            k = wl.k_cache[perm].contiguous()
+            v = wl.v_cache[perm].contiguous()
+        pools.append((k, v))
+    return pools
+
+
+def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="auto", waves=0, fuse=False):
+    """The decode step of a workload as a callable of the step index, plus its output and LSE tensors."""
+    B, Hq, D = wl.q.shape
+    out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
+    lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
+    # kv_split -1: the library chooses the split count and owns the partials
+    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev) if S > 0 else None
+    q_lens = [1] * B
+    kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=path, waves_per_block=waves, fuse_combine=fuse)
+    if wl.k_scale is not None:
+        kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
+    if wl.extra_out is not None:
+        kw.update(extra_partials=(wl.extra_out, wl.extra_lse))
+    if exact:
+        kw["plan_splits"] = False
+    fn = fd.gqa_fwd_batch_decode_persistent if variant == "persistent" else fd.gqa_fwd_batch_decode
+
+    def step(i):   # persistent: the scheduling launch is part of the step (inside the wrapper)
+        k, v = pools[i % len(pools)]
+        return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
+    return step, out, lse, workspace
+
+
+def settle(torch, step, ramp_ms):
+    """An idle GPU takes a while to reach its clocks, and a machine on which a process has just released tens of GiB
+    of device memory is busy with that for a few seconds more (measured: the first run after such a process read 5 %
+    slow, the same command seconds later did not).  Runs the step untimed, in batches timed with events, until the
+    batch time has settled (three batches in a row within 1 % of the best one) -- at least ramp_ms, at most 20 times
+    that.  Returns the milliseconds spent."""
+    t_ramp = time.perf_counter()
+    i_ramp, best, settled = 0, float("inf"), 0
+    r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    while ramp_ms > 0:
+        r0.record()
+        for _ in range(100):
+            step(i_ramp)
+            i_ramp += 1
+        r1.record()
+        torch.cuda.synchronize()
+        took = r0.elapsed_time(r1)
+        settled = settled + 1 if 0.99 * best <= took <= 1.01 * best else 0
+        best = min(best, took)
+        waited_ms = (time.perf_counter() - t_ramp) * 1e3
+        if (waited_ms >= ramp_ms and settled >= 3) or waited_ms >= 20 * ramp_ms:
+            break
+    return (time.perf_counter() - t_ramp) * 1e3
+
+
+def measure_target(torch, fd, dev, wl_cpu, steps, warmup, pools_n, ramp_ms, **step_kw):
+    """One north-star target measured the way the headline is: the whole decode step (split + combine) of a
+    workload, rotating over independent pools, after the clocks have settled.  Frees its pools on return."""
+    wl = wl_cpu.to(dev)
+    pools = make_pools(torch, wl, dev, pools_n)
+    step, _, _, _ = make_step(torch, fd, wl, pools, wl.kv_split, dev, **step_kw)
+    settle(torch, step, ramp_ms)
+    us = _time_us(torch, step, steps, warmup)
+    nbytes = wl_cpu.algorithmic_bytes()
+    del step, pools, wl
+    torch.cuda.empty_cache()
+    return {"us_per_step": round(us, 3), "algorithmic_bytes": nbytes,
+            "hbm_gbps_step": round(nbytes / (us * 1e-6) / 1e9, 1),
+            "frac_of_hbm_peak_step": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
+def measure_targets(torch, fd, dev, steps, warmup):
+    """Every north-star figure besides the headline, in this same process: config 2 with exactly the 32 splits the
+    workload names; config 5 (fp8 KV) and its bf16 twin, planned and with exactly 64 splits, and their ratios
+    (target >= 1.7); config 3; config 4 scheduled and unscheduled."""
+    U = fd.utils
+    t = {}
+    c2 = U.make_config(2)
+    t["config2_exact_32_splits"] = measure_target(torch, fd, dev, c2, steps, warmup, 4, 100.0, exact=True)
+    del c2
+    c5, c5t = U.make_config(5), U.make_config5_bf16_twin()
+    t["config5_fp8"] = measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0)
+    t["config5_fp8_exact_64_splits"] = measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0, exact=True)
+    t["config5_bf16_twin"] = measure_target(torch, fd, dev, c5t, steps, warmup, 4, 100.0)
+    t["config5_bf16_twin_exact_64_splits"] = measure_target(torch, fd, dev, c5t, steps, warmup, 4, 100.0, exact=True)
+    t["config5_bf16_over_fp8"] = round(t["config5_bf16_twin"]["us_per_step"] / t["config5_fp8"]["us_per_step"], 3)
+    t["config5_bf16_over_fp8_exact_64_splits"] = round(
+        t["config5_bf16_twin_exact_64_splits"]["us_per_step"] / t["config5_fp8_exact_64_splits"]["us_per_step"], 3)
+    del c5, c5t
+    c3 = U.make_config(3)
+    t["config3_sp_shard_plus_7_partials"] = measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0)
+    del c3
+    c4 = U.make_config(4)
+    n4 = max(5, steps // 4)   # a step of config 4 is 15 times config 2's
+    t["config4_ragged_scheduled"] = measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0, variant="persistent")
+    t["config4_ragged_unscheduled"] = measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0)
+    del c4
+    return t
 
 
 def measure_write_side(torch, fd, wl, dev, steps, warmup, decode_step, pools, kv_split):
@@ -218,61 +330,12 @@ def main():
     S = args.kv_split or wl.kv_split
     algo_bytes = wl_cpu.algorithmic_bytes()
 
-    # independent KV pools: pool 0 holds the seeded data (checked against the CPU baseline), the
-    # others hold other random bits of the same distribution
-    pools = [(wl.k_cache, wl.v_cache)]
-    for i in range(1, max(1, args.pools)):
-        if wl.k_cache.dtype in (torch.float16, torch.bfloat16, torch.float32):
-            k = torch.empty_like(wl.k_cache).normal_()
-            v = torch.empty_like(wl.v_cache).normal_()
-        else:  # fp8 bit patterns: shuffle pages of pool 0
-            perm = torch.randperm(wl.k_cache.shape[0], device=dev)
-            k = wl.k_cache[perm].contiguous()
-            v = wl.v_cache[perm].contiguous()
-        pools.append((k, v))
-
-    out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
-    lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
-    # kv_split -1: the library chooses the split count and owns the partials
-    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev) if S > 0 else None
-    q_lens = [1] * B
-    kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=args.path, waves_per_block=args.waves,
-              fuse_combine=args.fuse)
-    if wl.k_scale is not None:
-        kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
-    if wl.extra_out is not None:
-        kw.update(extra_partials=(wl.extra_out, wl.extra_lse))
-    if args.exact_splits:
-        kw["plan_splits"] = False
-    fn = fd.gqa_fwd_batch_decode_persistent if args.variant == "persistent" else fd.gqa_fwd_batch_decode
-
-    def step(i):   # persistent: the scheduling launch is part of the step (inside the wrapper)
-        k, v = pools[i % len(pools)]
-        return fn(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap, **kw)
+    pools = make_pools(torch, wl, dev, args.pools)
+    step, out, lse, workspace = make_step(torch, fd, wl, pools, S, dev, variant=args.variant, exact=args.exact_splits,
+                                          path=args.path, waves=args.waves, fuse=args.fuse)
 
     # ---- whole-step timing
-    # An idle GPU takes a while to reach its clocks, and a machine on which a process has just released tens of GiB of
-    # device memory is busy with that for a few seconds more (measured: the first run after such a process read 5 %
-    # slow, the same command seconds later did not).  Run the step untimed, in batches timed with events, until the
-    # batch time has settled (three batches in a row within 1 % of the best one) -- at least --clock-ramp-ms, at most
-    # 20 times that.
-    t_ramp = time.perf_counter()
-    i_ramp, best, settled = 0, float("inf"), 0
-    r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    while args.clock_ramp_ms > 0:
-        r0.record()
-        for _ in range(100):
-            step(i_ramp)
-            i_ramp += 1
-        r1.record()
-        torch.cuda.synchronize()
-        took = r0.elapsed_time(r1)
-        settled = settled + 1 if 0.99 * best <= took <= 1.01 * best else 0
-        best = min(best, took)
-        waited_ms = (time.perf_counter() - t_ramp) * 1e3
-        if (waited_ms >= args.clock_ramp_ms and settled >= 3) or waited_ms >= 20 * args.clock_ramp_ms:
-            break
-    ramp_ms = (time.perf_counter() - t_ramp) * 1e3
+    ramp_ms = settle(torch, step, args.clock_ramp_ms)
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -348,7 +411,7 @@ def main():
         del src, dst
     # HBM bytes per split-kernel launch from the committed counter runs (profiles/*__hbm_traffic.json,
     # FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None when this workload has none
-    traffic = None
+    traffic = traffic_source = None
     import glob
     candidates = [args.traffic_json] if args.traffic_json else sorted(
         glob.glob(os.path.join(ROOT, "profiles", "*__hbm_traffic.json")))
@@ -358,6 +421,7 @@ def main():
                 rec = json.load(f)
             if args.traffic_json or (rec.get("workload") == wl.name and args.path == "auto"):
                 traffic = rec.get("traffic")
+                traffic_source = os.path.relpath(path, ROOT)
                 break
 
     # ---- result of pool 0 for the check against the CPU baseline
@@ -392,7 +456,10 @@ def main():
         "clock_ramp_ms": round(ramp_ms),
         "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": traffic, "kernel_us": round(split_us, 3)},
+                     "traffic": traffic, "kernel_us": round(split_us, 3),
+                     # traffic is not measured by this run: it is the figure of the committed counter runs
+                     # (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, scaled by a copy of known size) for this workload
+                     "traffic_source": traffic_source},
     }
 
     # MFMA work of the split kernel (secondary figure: the path is HBM-bound).  Issued flops follow from the tiling:
@@ -412,6 +479,14 @@ def main():
         block = measure_decode_block(torch, fd, wl, dev, args.steps, args.warmup)
         if block is not None:
             result["decode_block"] = block
+
+    headline = args.config == 2 and not args.shape and not args.bf16_twin and args.variant == "plain" \
+        and not args.exact_splits and args.path == "auto" and not args.fuse and not args.kv_split
+    if headline and not args.no_targets:
+        del pools, step, workspace
+        wl = None
+        torch.cuda.empty_cache()
+        result["targets"] = measure_targets(torch, fd, dev, args.steps, args.warmup)
 
     if not args.no_cpu_baseline:
         import oracle  # the checker, timed as the CPU baseline only

@@ -103,6 +103,7 @@ constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
 constexpr int64_t kStoreThroughBytes = 16 << 20;   // partials of a step from which on they are written through
+constexpr int kMaxChunkBatch = 32;     // chunked work items: largest batch they are used for
 constexpr int kMaxSplitsPerWave = 2;   // chunked work items: splits one wave walks (all but the last parked in LDS)
 
 int env_waves() {
@@ -287,8 +288,10 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   // per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.
   a.chunk = 1;
   int chunk_wish = 1;
+  // Not for large batches: their lengths differ in practice, and many short work items balance better over the CUs
+  // than few long ones (config 4's ragged batch of 64 with exactly 32 splits: 691 us unchunked, 713 us chunked).
   if (use_mfma && D == 128 && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
-      !env_no_chunk()) {
+      batch <= kMaxChunkBatch && !env_no_chunk()) {
     fd_params plan = *p;
     plan.split_adapt = 0;
     const int s_plan = fd_plan_splits(&plan, batch);
