@@ -219,6 +219,34 @@ FD_API int fd_decode(void* stream, const void* q, const void* k_cache, const voi
               int32_t* tickets, const fd_params* params);
 
 /*
+ * fd_decode for callers that cannot allocate device memory -- code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose wrappers allocate
+ * their partial buffers with torch.empty on every call, flash_decode.py:783-786).  Same step and same kernels
+ * as fd_decode with tickets == NULL, but the split partials (fp32 [batch, Hq, num_splits, head_dim] and their
+ * LSEs, params->mid_dtype is ignored) live in a static device array inside the library instead of in
+ * out_split / lse_split; the call itself allocates nothing (no hipMalloc, no hipFree, no allocating library
+ * routine).  Limits and rules:
+ *   - batch * q_heads * num_splits * (head_dim + 1) * 4 bytes must not exceed FD_NOALLOC_SCRATCH_BYTES, else
+ *     FD_ERR_TOO_LARGE (nothing is launched); fd_plan_splits keeps all five benchmark configurations well
+ *     inside it;
+ *   - every GPU the library is used on holds its own copy of the array until the process ends;
+ *   - all calls on one GPU share that array: calls that may overlap on one GPU (different streams, graphs
+ *     replayed concurrently) race on it -- serialise them, or use fd_decode with workspaces of your own;
+ *     the array keeps the last call's partials, which the next call overwrites before it reads them.
+ */
+#define FD_NOALLOC_SCRATCH_BYTES (16u << 20)
+FD_API int fd_decode_noalloc(void* stream, const void* q, const void* k_cache, const void* v_cache,
+              void* out, float* lse_out, float sm_scale,
+              const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
+              int64_t stride_q_bs, int64_t stride_q_h,
+              int64_t stride_k_tok, int64_t stride_k_h,
+              int64_t stride_v_tok, int64_t stride_v_h,
+              int64_t stride_table_bs, int64_t stride_obs, int64_t stride_oh,
+              const int32_t* seq_order, int32_t combine_mode,
+              const void* extra_out, const float* extra_lse, int32_t num_extra,
+              const fd_params* params);
+
+/*
  * Kernel (3): work scheduler.  Writes seq_order[batch]: sequence indices sorted by
  * kv_len descending (ties by index), computed on the device from kv_lens, so that
  * fd_split_kv issues the longest sequences' workgroups first and the hardware

@@ -23,8 +23,9 @@ FD_F32, FD_F16, FD_BF16, FD_FP8_E4M3 = 0, 1, 2, 3
 FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
+FD_NOALLOC_SCRATCH_BYTES = 16 << 20   # static partial workspace of fd_decode_noalloc
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_decode_noalloc", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
                     "fd_kv_append",
                     "fd_last_error", "fd_abi_version")
 
@@ -101,6 +102,10 @@ def load_library(path: str = None) -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
         c_int32, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p,
         c_int32, c_void_p, POINTER(FdParams)]
+    lib.fd_decode_noalloc.restype = c_int32
+    lib.fd_decode_noalloc.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int32,
+        i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p, c_int32, POINTER(FdParams)]
     lib.fd_schedule_items.restype = c_int32
     lib.fd_schedule_items.argtypes = [c_void_p, c_void_p, c_int32, c_void_p, POINTER(FdParams)]
     lib.fd_plan_splits.restype = c_int32

@@ -147,6 +147,39 @@ int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_
 
 }  // namespace
 
+// Partial workspace of fd_decode_noalloc: a file-scope device array, so that the entry point never allocates.
+// Every GPU the library runs on holds its own copy (FD_NOALLOC_SCRATCH_BYTES of device memory until the process
+// ends) at its own address.  In host code the array's name is only a handle for the runtime, not a device
+// address: the address is looked up once per device with hipGetSymbolAddress and only that pointer is handed
+// to kernels.
+static __device__ __align__(256) unsigned char scratch[FD_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];   // per device, written once (every thread that races here writes the same value)
+
+// Device address of `scratch` on the current device, or nullptr with the error message set.
+void* scratch_on_current_device(const char* fn) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(FD_ERR_LAUNCH, "%s: hipGetDevice: %s (device %d)", fn, hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  void* ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (ptr) return ptr;
+  e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) {
+    fail(FD_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+    return nullptr;
+  }
+  __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+  return ptr;
+}
+
+}  // namespace
+
 extern "C" {
 const char* fd_last_error(void) { return g_err; }
 int fd_abi_version(void) { return FD_ABI_VERSION; }
@@ -456,6 +489,45 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
   return combine_impl(stream, out_split, lse_split, out, lse_out, kv_lens, batch, p->q_heads, p->num_splits,
                       stride_o_bs, stride_o_h, stride_o_split, stride_obs, stride_oh, combine_mode, extra_out,
                       extra_lse, num_extra, p, !skip_empty);
+}
+
+int fd_decode_noalloc(void* stream, const void* q, const void* k_cache, const void* v_cache, void* out, float* lse_out,
+                      float sm_scale, const int32_t* block_table, const int32_t* kv_lens, int32_t batch,
+                      int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok, int64_t stride_k_h,
+                      int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_table_bs, int64_t stride_obs,
+                      int64_t stride_oh, const int32_t* seq_order, int32_t combine_mode, const void* extra_out,
+                      const float* extra_lse, int32_t num_extra, const fd_params* p) {
+  const char* fn = "fd_decode_noalloc";
+  if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
+  if (batch < 0 || p->q_heads <= 0 || p->num_splits <= 0 || p->head_dim <= 0)
+    return fail(FD_ERR_INVALID_ARG, "%s: batch %d, q_heads %d, num_splits %d, head_dim %d", fn, batch, p->q_heads,
+                p->num_splits, p->head_dim);
+  const bool lse_twice = combine_mode == FD_COMBINE_SPLIT_LSE && lse_out;
+  if (p->num_splits == 1 && num_extra == 0 && !lse_twice)   // one split: written straight to `out`, no partials at all
+    return fd_decode(stream, q, k_cache, v_cache, nullptr, nullptr, out, lse_out, sm_scale, block_table, kv_lens, batch,
+                     stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h, 0, 0, 0,
+                     stride_table_bs, stride_obs, stride_oh, seq_order, combine_mode, extra_out, extra_lse, num_extra,
+                     nullptr, p);
+  // fp32 partials [batch, Hq, S, D] followed by their fp32 LSEs [batch, Hq, S]
+  const int64_t rows = (int64_t)batch * p->q_heads * p->num_splits;
+  const int64_t need = rows * (p->head_dim + 1) * 4;
+  if (need > (int64_t)FD_NOALLOC_SCRATCH_BYTES)
+    return fail(FD_ERR_TOO_LARGE,
+                "%s: batch %d x q_heads %d x num_splits %d x (head_dim %d + 1) fp32 partials = %lld bytes exceed the "
+                "static workspace of %lld bytes; use fewer splits (fd_plan_splits) or fd_decode with a workspace of "
+                "your own", fn, batch, p->q_heads, p->num_splits, p->head_dim, (long long)need,
+                (long long)FD_NOALLOC_SCRATCH_BYTES);
+  if (batch == 0) return FD_OK;
+  void* ws = scratch_on_current_device(fn);
+  if (!ws) return FD_ERR_LAUNCH;
+  fd_params own = *p;
+  own.mid_dtype = FD_F32;
+  const int64_t D = p->head_dim, S = p->num_splits;
+  float* lse_split = (float*)ws + rows * D;
+  return fd_decode(stream, q, k_cache, v_cache, ws, lse_split, out, lse_out, sm_scale, block_table, kv_lens, batch,
+                   stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h,
+                   (int64_t)p->q_heads * S * D, S * D, D, stride_table_bs, stride_obs, stride_oh, seq_order,
+                   combine_mode, extra_out, extra_lse, num_extra, nullptr, &own);
 }
 
 // Splits a shape needs to fill the chip, regardless of how long its sequences are (a power of two >= 1), or a

@@ -23,6 +23,9 @@ Keyword-only additions that the reference does not have (all default off):
                   and the library uses ``fd_plan_splits`` splits (same result, fewer workgroup prologues
                   and partials); False: exactly ``kv_split`` splits.  With a caller-supplied
                   ``output_split`` the split count and ranges are always the reference's.
+  no_alloc        True: the split partials live in the library's static device array (``fd_decode_noalloc``, at most
+                  16 MiB of them) and the call allocates nothing -- for steps captured into a HIP graph or run where
+                  allocation is not allowed; needs ``output_combine``; calls that overlap on one GPU must not share it
   fuse_combine    True: one launch, the combine runs in the tail of the split kernel (pays off when
                   the groups of a ragged batch finish at different times); False (default): split
                   kernel and combine kernel as two launches
@@ -40,7 +43,7 @@ from typing import Optional
 
 import torch
 
-from .._lib import (FD_BF16, FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F16, FD_F32, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
+from .._lib import (FD_BF16, FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F16, FD_F32, FD_NOALLOC_SCRATCH_BYTES, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
                     FdParams, check, fd_dtype_of, load_library, stream_handle)
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
@@ -194,7 +197,7 @@ def item_order_buffer(batch, num_splits, device):
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
             seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
-            schedule_items=False, item_order=None, max_kv_len=None):
+            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
@@ -227,7 +230,15 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         n_l = batch * q_heads * num_splits
         direct = (num_splits == 1 and extra_partials is None and not fuse_combine
                   and not (with_lse_column and lse_out is not None))
-        if direct:
+        if no_alloc:
+            # the partials live in the library's static device array (fd_decode_noalloc); nothing is allocated here
+            if output_combine is None or fuse_combine or schedule_items:
+                raise RuntimeError("no_alloc=True needs output_combine and neither fuse_combine nor a scheduling launch")
+            if n_o + n_l > FD_NOALLOC_SCRATCH_BYTES // 4:
+                raise RuntimeError(f"no_alloc=True: {4 * (n_o + n_l)} bytes of partials exceed the library's static "
+                                   f"workspace of {FD_NOALLOC_SCRATCH_BYTES} bytes")
+            hold = None
+        elif direct:
             # a single split: the split kernel writes the output itself, no partials and no combine launch
             hold = None
         elif (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
@@ -292,6 +303,17 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert ex_lse.is_contiguous() and ex_out.dtype == output_combine.dtype
     if lse_out is not None:
         assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
+    if no_alloc:
+        if output_split is not None:
+            raise RuntimeError("no_alloc=True keeps the partials inside the library; output_split cannot be given")
+        check(lib.fd_decode_noalloc(
+            hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_combine.data_ptr(),
+            lse_out.data_ptr() if lse_out is not None else None, float(scale), block_table.data_ptr(),
+            kv_lens.data_ptr(), batch, q_st[0], q_st[1], k_st[-3], k_st[-2], v_st[-3], v_st[-2], block_table.stride(0),
+            oc_st[0], oc_st[1], seq_order.data_ptr() if seq_order is not None else None,
+            FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
+            ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra, byref(p)))
+        return output_combine
     tickets = _tickets(q.device, hstream, batch * q_heads) if fuse_combine else None
     check(lib.fd_decode(
         hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), mid_ptr, lse_split_ptr,
