@@ -44,12 +44,36 @@ def assert_lse_close(lse, ref, rtol=LSE_RTOL):
     assert err.numel() == 0 or err.max().item() <= rtol, f"LSE rel err {err.max().item():.3e} > {rtol}"
 
 
-def assert_out_close(out, ref, atol=OUT_ATOL_16BIT, rtol=0.0):
+def assert_out_close(out, ref, atol=OUT_ATOL_16BIT, rtol=0.0, rel=True):
+    """The north-star gate (max-abs), and with ``rel`` the scale-aware gate below on top of it."""
     out, ref = out.float().cpu(), ref.float().cpu()
     assert torch.isfinite(out).all(), "non-finite output"
     err = (out - ref).abs()
     bound = atol + rtol * ref.abs()
     assert (err <= bound).all(), f"max abs err {err.max().item():.3e} (atol {atol}, rtol {rtol})"
+    if rel:
+        assert_out_rel(out, ref)
+
+
+# Scale-aware gate.  With thousands of N(0,1) value rows per sequence the outputs are 0.01-0.02 in magnitude, as large
+# as the north-star's absolute tolerance, so that gate alone would pass an output that is wrong by a constant factor.
+# Rounding the output to bf16 alone is 2^-9 relative per element (rms about 1.5e-3); 16-bit partials add as much again.
+OUT_RMS_RTOL = 1e-2        # rms(out - ref) / rms(ref)
+OUT_MAX_RTOL = 2e-2        # max|out - ref| / max|ref|
+
+
+def assert_out_rel(out, ref, rms_rtol=OUT_RMS_RTOL, max_rtol=OUT_MAX_RTOL):
+    """Error relative to the size of the reference values, per call (all elements together)."""
+    out, ref = out.double().cpu(), ref.double().cpu()
+    assert torch.isfinite(out).all(), "non-finite output"
+    if ref.numel() == 0 or not ref.any():
+        assert not out.any()
+        return
+    diff = out - ref
+    rms = (diff.pow(2).mean().sqrt() / ref.pow(2).mean().sqrt()).item()
+    mx = (diff.abs().max() / ref.abs().max()).item()
+    assert rms <= rms_rtol, f"rms error {rms:.3e} of the reference's rms (limit {rms_rtol})"
+    assert mx <= max_rtol, f"max error {mx:.3e} of the reference's largest value (limit {max_rtol})"
 
 
 def run_decode(fd, wl, variant="plain", **kw):
