@@ -168,7 +168,9 @@ FD_API int fd_split_kv(void* stream, const void* q, const void* k_cache, const v
  *            contiguous layout [batch, Hq, num_partials]
  *  out       [batch, Hq, D(+1)] params->out_dtype, strides stride_obs / stride_oh
  *  lse_out   NULL or fp32 [batch, Hq]: merged natural-log LSE (always fp32)
- *  seqlens   kv_lens [batch] (split modes) or global_kv_lens [num_partials, batch] (rank mode)
+ *  seqlens   kv_lens [batch] (split modes) or global_kv_lens [num_partials, batch] (rank mode).  In the
+ *            split modes a length is clamped to params->max_pages_per_seq * params->page_size when both
+ *            are set, exactly as the split kernels clamp it, so both agree on which ranges exist.
  *  extra_out / extra_lse / num_extra
  *            further always-valid partials merged in the same pass:
  *            extra_out [num_extra, batch, Hq, D] contiguous in params->out_dtype,
@@ -365,6 +367,14 @@ FD_API const char* fd_last_error(void);
 
 /* FD_ABI_VERSION the library was built with. */
 FD_API int fd_abi_version(void);
+
+/*
+ * Identifies the sources the library was built from: the build script passes a hash of every source and header
+ * (FD_BUILD_ID), "unknown" for a build made some other way.  A loader compares it with the hash of the sources
+ * it sees to detect a stale library (triton-distributed_amd/build.py::ensure_built).  No counterpart in the
+ * reference.
+ */
+FD_API const char* fd_build_id(void);
 
 #ifdef __cplusplus
 }

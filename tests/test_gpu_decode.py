@@ -693,6 +693,44 @@ def test_short_sequences_in_a_block_table_sized_for_long_contexts(fd, capacity, 
     assert_lse_close(res[..., D].float(), ref_lse, rtol=1e-5 if f32 else 1e-2)
 
 
+def test_lengths_above_the_table_capacity_are_clamped_alike_by_split_and_combine(fd):
+    """kv_lens beyond max_pages * page_size are documented as clamped to the capacity.  With more than 16 splits and
+    ranges by each sequence's own length the empty ranges write nothing and the combine derives the valid slots from
+    kv_lens: it has to clamp the way the split kernels do, or it would merge slots that nobody wrote."""
+    P, cap_pages = 16, 512          # capacity 8192 tokens
+    lens_real = [8192, 8192, 3000]
+    wl = fd.utils.make_paged_workload("over_capacity", lens_real, 32, 8, 128, P, torch.bfloat16, 32, seed=37)
+    assert wl.block_table.shape[1] == cap_pages
+    ref, ref_lse = oracle_decode(wl)
+    wl.kv_lens = torch.tensor([100000, 8193, 3000], dtype=torch.int32)   # two of them above the capacity
+    g = wl.to(DEV)
+    B, Hq, D = g.q.shape
+    for kv_split, adapt in ((32, 2), (64, 1), (32, 0)):
+        lse = torch.empty(B, Hq, dtype=torch.float32, device=DEV)
+        out = torch.empty(B, Hq, D, dtype=g.q.dtype, device=DEV)
+        # poison the partial workspace: a slot that is read without having been written shows
+        ws = torch.full((B * Hq * kv_split * (D + 1),), float("nan"), dtype=torch.float32, device=DEV)
+        L = fd._lib
+        lib = fd.load_library()
+        p = L.FdParams()
+        p.q_heads, p.kv_heads, p.head_dim, p.page_size = Hq, 8, D, P
+        p.num_splits, p.num_pages, p.max_pages_per_seq = kv_split, g.k_cache.shape[0], cap_pages
+        p.q_dtype = p.kv_dtype = p.out_dtype = L.FD_BF16
+        p.mid_dtype = L.FD_F32
+        p.split_align, p.split_adapt = (64, adapt) if adapt else (0, 0)
+        from ctypes import byref
+        n_o = B * Hq * kv_split * D
+        L.check(lib.fd_decode(
+            torch.cuda.current_stream().cuda_stream, g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(),
+            ws.data_ptr(), ws.data_ptr() + 4 * n_o, out.data_ptr(), lse.data_ptr(), float(g.scale),
+            g.block_table.data_ptr(), g.kv_lens.data_ptr(), B, g.q.stride(0), g.q.stride(1), g.k_cache.stride(-3),
+            g.k_cache.stride(-2), g.v_cache.stride(-3), g.v_cache.stride(-2), Hq * kv_split * D, kv_split * D, D,
+            g.block_table.stride(0), out.stride(0), out.stride(1), None, 0, None, None, 0, None, byref(p)))
+        torch.cuda.synchronize()
+        assert_out_close(out.cpu(), ref)
+        assert_lse_close(lse.cpu(), ref_lse)
+
+
 # ---- scheduled issue order by (sequence, range) items: the scheduling launch, the append-fused one, the raw ABI
 @pytest.mark.parametrize("capacity", [4096, 65536])
 @pytest.mark.parametrize("kind", ["bf16", "fp8", "fp32_valu"])

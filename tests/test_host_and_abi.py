@@ -238,3 +238,19 @@ def test_split_plan_policy(fd):
         assert 1 <= got <= args[3]
     assert plan(0, 32, 8, 32, 512) < 0 and b"fd_plan_splits" in lib.fd_last_error()
     assert lib.fd_plan_splits(None, 1) < 0
+
+
+def test_a_stale_library_is_rebuilt_not_silently_used(fd, monkeypatch):
+    """ensure_built() compares the build id inside the library with the hash of the sources beside it."""
+    import importlib
+    b = importlib.import_module("triton-distributed_amd.build")
+    assert b.built_id() == b.source_id() == fd.load_library().fd_build_id().decode()
+    assert b.ensure_built() == b.LIB_PATH           # up to date: used as it is
+    calls = []
+    monkeypatch.setattr(b, "source_id", lambda: "0123456789abcdef")          # as if a source had been edited
+    monkeypatch.setattr(b, "build", lambda force=False, verbose=True: calls.append(force) or b.LIB_PATH)
+    with pytest.raises(RuntimeError, match="does not match the sources"):
+        b.ensure_built()                            # the (stubbed) rebuild did not produce a matching library
+    assert calls == [True]
+    monkeypatch.setenv("FD_LIBRARY_PATH", "/somewhere/else.so")            # an explicit library is the caller's business
+    assert b.ensure_built() == "/somewhere/else.so"

@@ -27,7 +27,7 @@ FD_NOALLOC_SCRATCH_BYTES = 16 << 20   # static partial workspace of fd_decode_no
 
 EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_decode_noalloc", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
                     "fd_kv_append",
-                    "fd_last_error", "fd_abi_version")
+                    "fd_last_error", "fd_abi_version", "fd_build_id")
 
 _DTYPES = {torch.float32: FD_F32, torch.float16: FD_F16, torch.bfloat16: FD_BF16}
 if hasattr(torch, "float8_e4m3fn"):
@@ -122,6 +122,8 @@ def load_library(path: str = None) -> ctypes.CDLL:
     lib.fd_last_error.argtypes = []
     lib.fd_abi_version.restype = c_int32
     lib.fd_abi_version.argtypes = []
+    lib.fd_build_id.restype = c_char_p
+    lib.fd_build_id.argtypes = []
     if lib.fd_abi_version() != FD_ABI_VERSION:
         raise RuntimeError(f"{path}: ABI version {lib.fd_abi_version()} != expected {FD_ABI_VERSION}; rebuild")
     _lib = lib

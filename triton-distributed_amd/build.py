@@ -9,6 +9,7 @@ source tree; nothing is installed into site-packages.
 from __future__ import annotations
 
 import argparse
+import hashlib
 import os
 import shutil
 import subprocess
@@ -47,11 +48,40 @@ def _stale(target: str, deps) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def _compile(src: str, force: bool, verbose: bool) -> str:
+def source_id() -> str:
+    """Hash of every source and header the library is built from (and of the compiler flags)."""
+    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    for path in [os.path.join(CSRC, s) for s in SOURCES] + HEADERS:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+_ID_TAG = b"FD_BUILD_ID="
+
+
+def built_id(path: str = LIB_PATH) -> str:
+    """The build id inside a built library (what its ``fd_build_id()`` returns), read from the file without loading
+    it -- a stale image, once loaded, would stay this process's image of that path; "" if there is none."""
+    try:
+        with open(path, "rb") as f:
+            blob = f.read()
+    except OSError:
+        return ""
+    at = blob.find(_ID_TAG)
+    if at < 0:
+        return ""
+    end = blob.find(b"\0", at)
+    return blob[at + len(_ID_TAG):end].decode("ascii", "replace")
+
+
+def _compile(src: str, force: bool, verbose: bool, build_id: str) -> str:
     obj = os.path.join(BUILD, os.path.splitext(src)[0] + ".o")
     path = os.path.join(CSRC, src)
-    if force or _stale(obj, [path] + HEADERS):
-        cmd = [_hipcc()] + HIPCC_FLAGS + ["-c", path, "-o", obj]
+    stamped = src == "fd_api.hip"   # the translation unit that carries the build id: rebuilt whenever the id changes
+    if force or _stale(obj, [path] + HEADERS) or stamped:
+        cmd = [_hipcc()] + HIPCC_FLAGS + ([f'-DFD_BUILD_ID="{build_id}"'] if stamped else []) + ["-c", path, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -68,8 +98,9 @@ def _compile(src: str, force: bool, verbose: bool) -> str:
 def build(force: bool = False, verbose: bool = True) -> str:
     """Compiles every HIP source for gfx950 and links the shared library.  Returns its path."""
     os.makedirs(BUILD, exist_ok=True)
+    build_id = source_id()
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), 8)) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force, verbose), SOURCES))
+        objs = list(ex.map(lambda s: _compile(s, force, verbose, build_id), SOURCES))
     if force or _stale(LIB_PATH, objs):
         cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
         if verbose:
@@ -90,11 +121,22 @@ if __name__ == "__main__":
 
 
 def ensure_built(verbose: bool = False) -> str:
-    """For tests, the smoke check and the bench: the library as it is if it has been built (or FD_LIBRARY_PATH names
-    one), else one build.  The package itself never builds behind the caller's back: ``load_library`` raises."""
+    """For tests, the smoke check and the bench: the library as it is if it has been built from the sources in this
+    tree (or FD_LIBRARY_PATH names one), else one build.  A library whose ``fd_build_id()`` differs from the hash of
+    the sources beside it is stale -- it would be tested in place of the code under review -- and is rebuilt (an
+    error if that is not possible, never a silent pass).  The package itself never builds behind the caller's
+    back: ``load_library`` raises."""
     override = os.environ.get("FD_LIBRARY_PATH")
     if override:
         return override
     if os.path.exists(LIB_PATH):
+        want, have = source_id(), built_id()
+        if have == want:
+            return LIB_PATH
+        print(f"{LIB_NAME} is stale (built from {have or 'unknown sources'}, the tree is {want}): rebuilding",
+              file=sys.stderr, flush=True)
+        build(force=True, verbose=verbose)
+        if built_id() != want:
+            raise RuntimeError(f"{LIB_PATH} does not match the sources after a rebuild")
         return LIB_PATH
     return build(force=False, verbose=verbose)

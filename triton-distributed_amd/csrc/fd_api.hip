@@ -183,6 +183,12 @@ void* scratch_on_current_device(const char* fn) {
 extern "C" {
 const char* fd_last_error(void) { return g_err; }
 int fd_abi_version(void) { return FD_ABI_VERSION; }
+#ifndef FD_BUILD_ID
+#define FD_BUILD_ID "unknown"
+#endif
+// kept with its tag so that the id can also be read from the file without loading it
+static const char g_build_id[] = "FD_BUILD_ID=" FD_BUILD_ID;
+const char* fd_build_id(void) { return g_build_id + sizeof("FD_BUILD_ID=") - 1; }
 }
 
 namespace {
@@ -639,6 +645,13 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
                   a.adapt, num_partials);
   }
   div_magic((uint32_t)num_partials, &a.s_magic, &a.s_shift);
+  // Lengths beyond the block table's capacity are clamped exactly as the split kernels clamp them, so that both
+  // agree on which ranges exist; a caller that names no table still gets kv_len + num_partials - 1 < 2^31.
+  a.capacity = ((int64_t)1 << 31) - 1 - num_partials;
+  if (p->max_pages_per_seq > 0 && p->page_size > 0) {
+    const int64_t cap = (int64_t)p->max_pages_per_seq * p->page_size;
+    if (cap < a.capacity) a.capacity = cap;
+  }
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;

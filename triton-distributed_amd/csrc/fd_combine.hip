@@ -56,7 +56,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   const bool own = a.all_slots_written && a.mode != FD_COMBINE_RANK;
   int kv_len = 0, per = 0;
   if (a.mode != FD_COMBINE_RANK && !own) {
-    kv_len = max(a.seqlens[b], 0);
+    kv_len = (int)min((int64_t)max(a.seqlens[b], 0), a.capacity);   // the length the split kernels worked with
     per = tokens_per_range(kv_len, S, a.s_magic, a.s_shift, a.per_mask, a.adapt);
   }
   // LSE of partial s, -inf when the partial is not valid

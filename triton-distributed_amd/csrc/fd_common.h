@@ -93,6 +93,8 @@ struct CombineArgs {
   uint32_t s_magic, s_shift;  // n / num_partials, as in SplitArgs
   int32_t all_slots_written;  // 1: the partials come from this library's split kernel in the same call, which
                               // writes every slot (empty splits as out = 0, lse = -inf)
+  int64_t capacity;           // split modes: lengths are clamped to it, as the split kernels clamp them to the block
+                              // table's capacity (stand-alone calls that do not know a table: 2^31 - 1 - num_partials)
 };
 
 // How a decode step cuts a sequence into ranges: what the scheduler needs to know of it.

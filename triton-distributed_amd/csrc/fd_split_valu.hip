@@ -262,6 +262,11 @@ int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
     const size_t need = (size_t)(a.S + a.num_extra) * gh * 4;
     if (need > lds) lds = need;
   }
+  if (lds > 64 * 1024) {
+    // more than the default 64 KB of dynamic LDS per workgroup (gfx950 has 160 KB per CU)
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return FD_ERR_LAUNCH;
+  }
   hipLaunchKernelGGL(kern, grid, dim3(block), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }

@@ -53,8 +53,11 @@ MAX_AUTO_KV_SPLITS = 256  # upper bound of the library's own choice (kv_split ==
 
 
 def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size, split_kv=32, soft_cap=0.0):
-    """Meta-parameters of the split kernel, the counterpart of ``get_triton_split_kv_algo_info``
-    (flash_decode.py:103-109): what the gfx950 kernels use instead of BLOCK_N/BLOCK_H/num_warps."""
+    """Counterpart of ``get_triton_split_kv_algo_info`` (flash_decode.py:103-109).  There the dictionary selects an
+    ahead-of-time compiled Triton kernel; here it is informational only -- nothing in this package reads it back:
+    the library is compiled for every supported combination and picks kernel, tile, waves per workgroup and work
+    items per call inside ``fd_split_kv`` / ``fd_decode`` (``fd_plan_splits`` reports the split count it would use).
+    The entries describe the kernel family a shape runs on: token tile, query heads per wave, wave size."""
     group = q_heads // kv_heads
     mfma = q_head_dim in (64, 128, 256)   # 16-bit / fp8 caches; fp32 caches run on the VALU kernel
     return {
@@ -69,7 +72,8 @@ get_triton_split_kv_algo_info = get_split_kv_algo_info  # reference name (kernel
 
 
 def get_combine_kv_algo_info(split_kv=32, v_head_dim=128, block_dv=512):
-    """Counterpart of ``get_triton_combine_kv_algo_info`` (flash_decode.py:281-285)."""
+    """Counterpart of ``get_triton_combine_kv_algo_info`` (flash_decode.py:281-285); informational only, like
+    ``get_split_kv_algo_info``: ``fd_combine`` chooses its own launch shape."""
     return {"NUM_KV_SPLITS": split_kv, "Lv": v_head_dim, "BLOCK_DV": block_dv, "wave_size": 64, "waves": 1}
 
 

@@ -1,63 +1,21 @@
 """KV caches for the decode block.
 
-``KV_Cache`` has the constructor, attributes and methods of the reference's dense cache
-(``python/triton_dist/models/kv_cache.py:28-69``): ``[layers, B, max_length, Hkv/world, D]`` plus an int32
-``kv_offset [B]``.  Its per-layer slice is what ``flash_attn_with_kvcache`` takes as a dense cache: one
-"page" of ``max_length`` tokens per sequence.
-
 ``PagedKV_Cache`` is the layout the decode path is built for (``[pages, P, Hkv, D]`` pools with an int32
 block table, python/triton_dist/test/nvidia/test_decode_attn.py:150-156), optionally fp8-e4m3 with
 per-KV-head scales; the reference has no paged owner class, so this one only adds what the kernels need:
-the pools, a block table and the same ``kv_offset`` bookkeeping.
+the pools, a block table and the ``kv_offset`` bookkeeping.
+
+``KV_Cache`` is the reference's dense cache (``python/triton_dist/models/kv_cache.py:28-69``:
+``[layers, B, max_length, Hkv/world, D]`` plus an int32 ``kv_offset [B]``) expressed in that layout: one page of
+``max_length`` tokens per sequence with the identity block table, so a layer's slice ``[B, max_length, Hkv, D]`` is
+both what the reference's attention call takes as a dense cache and a valid pool for the paged kernels.  It keeps
+the reference's constructor arguments, attribute names and methods so the decode block reads the same.
 """
 from __future__ import annotations
 
 from typing import Optional
 
 import torch
-
-
-class KV_Cache:
-
-    def __init__(self, num_layers: int = 32, batch_size: int = 1, max_length: int = 32 * 1024, kv_heads: int = 8,
-                 head_dim: int = 128, dtype=torch.bfloat16, world_size: int = 8) -> None:
-        self.num_layers = num_layers
-        self.batch_size = batch_size
-        self.max_length = max_length
-        self.kv_heads = kv_heads
-        self.head_dim = head_dim
-        self.dtype = dtype
-        self.world_size = world_size
-        shape = (num_layers, batch_size, max_length, kv_heads // world_size, head_dim)
-        self.k_cache = torch.zeros(shape, device="cuda", dtype=self.dtype)
-        self.v_cache = torch.zeros(shape, device="cuda", dtype=self.dtype)
-        self.kv_offset = torch.zeros(batch_size, dtype=torch.int32, device="cuda")
-
-    def update_kv_cache(self, new_k_cache: torch.Tensor, new_v_cache: torch.Tensor, layer_idx: int):
-        """Returns the layer's caches and the offsets; the new token is written by the attention call
-        (models/kv_cache.py:46-47)."""
-        return self.k_cache[layer_idx], self.v_cache[layer_idx], self.kv_offset
-
-    def rand_fill_kv_cache(self, offset: int):
-        kv_shape = self.k_cache[:, :, :offset].size()
-        k = torch.rand(kv_shape, device="cuda", dtype=self.dtype) / 10
-        v = torch.rand(kv_shape, device="cuda", dtype=self.dtype) / 10
-        self.k_cache[:, :, :offset].copy_(k)
-        self.v_cache[:, :, :offset].copy_(v)
-
-    def inc_offset(self):
-        self.kv_offset += 1
-
-    def clear(self):
-        self.kv_offset.zero_()
-
-    def get_kv_len(self):
-        return self.kv_offset
-
-    # what flash_attn_with_kvcache needs besides the slices: nothing (a dense cache has an implicit table)
-    block_table = None
-    k_scale = None
-    v_scale = None
 
 
 class PagedKV_Cache:
@@ -118,3 +76,21 @@ class PagedKV_Cache:
 
     def get_kv_len(self):
         return self.kv_offset
+
+
+class KV_Cache(PagedKV_Cache):
+    """Dense cache = ``PagedKV_Cache`` with ``page_size == max_length`` and pages in sequence order."""
+
+    def __init__(self, num_layers: int = 32, batch_size: int = 1, max_length: int = 32 * 1024, kv_heads: int = 8,
+                 head_dim: int = 128, dtype=torch.bfloat16, world_size: int = 8) -> None:
+        super().__init__(num_layers=num_layers, batch_size=batch_size, max_length=max_length, kv_heads=kv_heads,
+                         head_dim=head_dim, dtype=dtype, world_size=world_size, page_size=max_length, fp8=False,
+                         shuffle=False)
+        # the attention call derives the table of a dense cache itself ([b] -> page b)
+        self.block_table = None
+
+    def rand_fill_kv_cache(self, offset: int):
+        """Uniform values in [0, 0.1) in the first ``offset`` positions of every layer and sequence (the range the
+        reference's benchmark fill uses, models/kv_cache.py:52-57); ``kv_offset`` is left alone, as there."""
+        for cache in (self.k_cache, self.v_cache):
+            cache[:, :, :offset].uniform_(0.0, 0.1)

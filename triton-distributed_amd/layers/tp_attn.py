@@ -21,9 +21,11 @@ from ..kernels.kv_append import flash_attn_with_kvcache
 
 
 def layer_norm(hidden_states: torch.Tensor, eps: float, w: torch.Tensor):
-    """RMS norm over the last dimension (tp_attn.py:52-59)."""
-    return nn.functional.rms_norm(hidden_states.view(-1, hidden_states.size(-1)),
-                                  normalized_shape=(hidden_states.size(-1), ), weight=w, eps=eps).view_as(hidden_states)
+    """Per-row RMS norm over the last dimension with weight ``w``: the reference's helper of this name
+    (tp_attn.py:52-59), used on q and k when the model has q_norm / k_norm."""
+    width = hidden_states.shape[-1]
+    rows = hidden_states.reshape(-1, width)
+    return nn.functional.rms_norm(rows, (width,), w, eps).reshape(hidden_states.shape)
 
 
 def _set_cos_sin_cache(inv_freq: torch.Tensor, max_length: int):

@@ -18,17 +18,18 @@ import torch
 
 
 def perf_func(func, iters, warmup_iters):
-    start_event = torch.cuda.Event(enable_timing=True)
-    stop_event = torch.cuda.Event(enable_timing=True)
-    output = None
-    for n in range(iters + warmup_iters):
-        if n == warmup_iters:
-            start_event.record()
-        output = func()
-    stop_event.record()
-    torch.cuda.current_stream().synchronize()
-    duration_ms = start_event.elapsed_time(stop_event)
-    return output, duration_ms / iters
+    """``(last result, mean milliseconds per call)`` of ``iters`` back-to-back calls after ``warmup_iters`` untimed
+    ones, timed by two events on the current stream -- the reference's method and signature (utils.py:269-281)."""
+    result = None
+    for _ in range(warmup_iters):
+        result = func()
+    begin, end = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+    begin.record()
+    for _ in range(iters):
+        result = func()
+    end.record()
+    end.synchronize()
+    return result, begin.elapsed_time(end) / iters
 
 
 @dataclasses.dataclass
