@@ -86,6 +86,53 @@ def test_sp_layer_matches_oracle_on_concatenated_cache(fd, R, Hq, Hkv, P, dtype)
         layer.finalize()
 
 
+def test_sp_layer_at_the_reference_settings_200_iterations(fd):
+    """The reference's own loop (test_sp_decode_attn.py:158-202): 96 / 12 heads, head_dim 128, page size 1, fp16,
+    1536 tokens per rank, K/V ~ N(0,1)/10, fresh seeded inputs in each of 200 iterations, the oracle on the
+    concatenated cache, atol 0.05 / rtol 1e-2 -- with the layer at the reference's settings: 32 splits, split
+    partials the caller can see, and everything staged in the query's dtype (LSE included, :95-97), over a
+    3-stage ring.  All "ranks" run on the one GPU; every rank's partial comes from the same call the layer makes."""
+    R, B, Hq, Hkv, D, P, n, dtype = 4, 1, 96, 12, 128, 1, 128 * 12, torch.float16
+    pages = n + 1
+    scale = D ** -0.5
+    rank = 1
+    layer = fd.SpGQAFlashDecodeAttention(rank, 0, R, 1, Hq, Hkv, D, D, page_size=P, scale=scale, soft_cap=0,
+                                         max_allowed_batch=1, thrink_buffer_threshold=500, stages=3,
+                                         partial_dtype=None)
+    layer.kv_split = 32
+    gen = torch.Generator(device=DEV).manual_seed(2024)
+    lens = torch.full((R, B), n, dtype=torch.int32, device=DEV)
+    worst = 0.0
+    for it in range(200):
+        q = torch.randn(B, Hq, D, generator=gen, device=DEV, dtype=torch.float32).to(dtype)
+        kv = (torch.randn(R, 2, pages, P, Hkv, D, generator=gen, device=DEV, dtype=torch.float32) / 10).to(dtype)
+        bts = torch.randint(0, pages, (R, B, pages), generator=gen, device=DEV, dtype=torch.int32)
+        parts = []
+        for r in range(R):
+            if r == rank:
+                continue
+            mid = torch.empty(B, Hq, 32, D + 1, dtype=dtype, device=DEV)
+            oc = torch.empty(B, Hq, D + 1, dtype=dtype, device=DEV)
+            fd.gqa_fwd_batch_decode_intra_rank(q, kv[r, 0], kv[r, 1], None, [1] * B, lens[r], bts[r], scale,
+                                               output_split=mid, output_combine=oc, kv_split=32)
+            parts.append(oc)
+        r_out = torch.stack([p_[..., :D] for p_ in parts])
+        r_lse = torch.stack([p_[..., D].float() for p_ in parts])
+        output_split = torch.full((B, Hq, 32, D + 1), float("nan"), dtype=dtype, device=DEV)
+        out = layer(q, kv[rank, 0], kv[rank, 1], lens, bts[rank], remote_partials=(r_out, r_lse),
+                    output_split=output_split)
+        torch.cuda.synchronize()
+        assert not torch.isnan(output_split).any()        # all 32 partials of every head were written
+        kv_c, bts_c = kv.cpu(), bts.cpu()
+        ref, _ = _oracle_concat(q.cpu(), [kv_c[r, 0] for r in range(R)], [kv_c[r, 1] for r in range(R)],
+                                [bts_c[r] for r in range(R)], lens.cpu(), pages, scale)
+        torch.testing.assert_close(out.float().cpu(), ref, atol=0.05, rtol=1e-2)
+        worst = max(worst, (out.float().cpu() - ref).abs().max().item())
+    assert layer.signal_target == 200
+    assert worst < 5e-3, worst      # far inside the reference's tolerance: fp16 partials and LSEs of values ~0.01
+    layer.finalize()
+
+
 def test_sp_layer_single_rank_and_reference_partial_dtype(fd):
     q, ks, vs, bts, lens, pages = _sp_inputs(1, 1, 32, 8, 128, 16, [[777]], torch.bfloat16, seed=9, scale_kv=1.0)
     ref, _ = _oracle_concat(q, ks, vs, bts, lens, pages, 0.09)

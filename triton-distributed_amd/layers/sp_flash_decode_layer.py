@@ -53,7 +53,8 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         self.soft_cap = soft_cap
         self.scale = scale
         # The reference fixes 32 splits (sp_flash_decode_layer.py:62).  The partials never leave this layer, so the
-        # count is left to the library: 32 for short shards, up to 256 for long ones.
+        # count is left to the library: 32 for short shards, up to 256 for long ones.  Set it to 32 (and pass
+        # ``partial_dtype=None``) for the reference's settings.
         self.kv_split = -1
         self.max_allowed_batch = max_allowed_batch
         self.stages = stages
@@ -91,13 +92,16 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         return self.ag_buffer[self.signal_target % self.stages][:nbytes]
 
     def forward(self, q, k_cache, v_cache, global_kv_lens, block_table,
-                remote_partials: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+                remote_partials: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                output_split: Optional[torch.Tensor] = None):
         """
         q: each rank has the same q
         k_cache / v_cache: this rank's shard of the paged cache
         global_kv_lens: [num_ranks, B] int32, every rank's local kv length
         block_table: this rank's block table
         remote_partials: the other ranks' (out, lse), see the module docstring
+        output_split: optional caller-visible split partials ``[B, Hq, kv_split, Dv+1]`` as the reference allocates
+            them on every call (:95-96); needs ``self.kv_split`` set to that split count (the reference's is 32)
         """
         batch = q.shape[0]
         assert global_kv_lens.shape[0] == self.num_ranks
@@ -118,6 +122,7 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         # local decode straight into this rank's slot (the reference copies it there, :136-138)
         gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch, global_kv_lens[self.rank],
                                         block_table, self.scale, soft_cap=self.soft_cap,
+                                        output_split=output_split,
                                         output_combine=all_ranks_output_combine[self.rank], kv_split=self.kv_split)
 
         # stand-in for the allgather: the other ranks' partials arrive from the caller
