@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FD_ABI_VERSION 1
+#define FD_ABI_VERSION 2
 
 #if defined(__GNUC__)
 #define FD_API __attribute__((visibility("default")))
@@ -77,7 +77,8 @@ typedef enum fd_combine_mode {
 typedef struct fd_params {
   int32_t q_heads;          /* Hq                                                  */
   int32_t kv_heads;         /* Hkv; Hq % Hkv == 0                                  */
-  int32_t head_dim;         /* Dk == Dv; 64, 128 or 256                            */
+  int32_t head_dim;         /* Dk (= the query's head dim); 64, 128 or 256; also Dv
+                               unless v_head_dim says otherwise                    */
   int32_t page_size;        /* tokens per page (any value >= 1)                    */
   int32_t num_splits;       /* NUM_KV_SPLITS                                       */
   int32_t num_pages;        /* pages in the pool: table entries are clamped to
@@ -119,6 +120,12 @@ typedef struct fd_params {
   int32_t seq_order_items;  /* 0: seq_order / seq_order_out is a per-sequence order ([batch], see
                                fd_schedule and fd_kv_append).  1: it is the work-item order of
                                fd_schedule_items, int32 [2 * batch * num_splits].             */
+  int32_t v_head_dim;       /* 0: Dv = head_dim.  Else 64, 128 or 256: the V cache's head dim, which the
+                               reference takes from the V cache independently of K's (V_DIM next to K_DIM,
+                               flash_decode.py:162-163, 765-774).  Partials and outputs then have Dv (+1)
+                               columns and fd_combine works on Dv.  Dv != Dk runs on the VALU kernel
+                               (fp32 / fp16 / bf16 caches; FD_ERR_UNSUPPORTED with FD_PATH_MFMA, with an
+                               fp8 cache and in fd_kv_append).                                  */
 } fd_params;
 
 /*

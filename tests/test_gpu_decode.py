@@ -69,6 +69,47 @@ def test_head_dim_64(fd, dtype, num_heads, block_size, soft_cap):
     assert_lse_close(lse_m, ref_lse)
 
 
+# ---- V head dim != K head dim (flash_decode.py:765-774 takes v_head_dim from the V cache; K_DIM / V_DIM :162-163)
+@pytest.mark.parametrize("dims", [(128, 64), (128, 256), (64, 128), (256, 64), (64, 256), (256, 128)])
+@pytest.mark.parametrize("dtype,num_heads,block_size,soft_cap", [
+    (torch.bfloat16, (32, 8), 16, 0), (torch.float16, (6, 1), 1, 30), (torch.float32, (16, 16), 7, 0),
+    (torch.bfloat16, (20, 2), 16, 50)])
+def test_v_head_dim_differs_from_k_head_dim(fd, dims, dtype, num_heads, block_size, soft_cap):
+    Dk, Dv = dims
+    wl = _grid_workload(fd, [1320, 18, 463, 1, 0, 70, 2500], num_heads, Dk, block_size, dtype, soft_cap, seed=Dk + Dv)
+    gen = torch.Generator().manual_seed(Dk * 7 + Dv)
+    wl.v_cache = torch.randn(*wl.k_cache.shape[:3], Dv, generator=gen).to(dtype)
+    ref, ref_lse = oracle_decode(wl)
+    assert ref.shape[-1] == Dv
+    f32 = dtype == torch.float32
+    tol = dict(atol=2e-4 if f32 else 2e-2)
+    for kw in (dict(), dict(plan_splits=False), dict(fuse_combine=True), dict(variant="persistent"),
+               dict(waves_per_block=2, plan_splits=False)):
+        out, lse = run_decode(fd, wl, **kw)
+        assert out.shape[-1] == Dv
+        assert_out_close(out, ref, **tol)
+        assert_lse_close(lse, ref_lse, rtol=1e-5 if f32 else 1e-3)
+    # merged LSE at column Dv, and caller-visible partials [B, Hq, S, Dv + 1] against the per-split model
+    res, _ = run_decode(fd, wl, variant="intra")
+    assert res.shape[-1] == Dv + 1
+    assert_out_close(res[..., :Dv], ref, **tol)
+    assert_lse_close(res[..., Dv].float(), ref_lse, rtol=1e-5 if f32 else 1e-2)
+    B, Hq = wl.q.shape[:2]
+    mid = torch.full((B, Hq, 8, Dv + 1), float("nan"), dtype=torch.float32, device=DEV)
+    wl.kv_split = 8
+    out_v, _ = run_decode(fd, wl, output_split=mid)
+    assert_out_close(out_v, ref, **tol)
+    model = oracle.model_split_kv(wl.q.float(), wl.k_cache.float(), wl.v_cache.float(), wl.kv_lens.tolist(),
+                                  wl.block_table, wl.scale, 8, soft_cap=wl.soft_cap)
+    valid = torch.isfinite(model[..., Dv])
+    got = mid.cpu()
+    assert torch.allclose(got[..., :Dv][valid], model[..., :Dv][valid], atol=2e-5 if f32 else 2e-3)
+    assert torch.allclose(got[..., Dv][valid], model[..., Dv][valid], atol=1e-3, rtol=1e-3)
+    if not f32:   # the MFMA kernels need equal dims and say so
+        with pytest.raises(RuntimeError, match="equal K and V head"):
+            run_decode(fd, wl, path="mfma")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("num_heads", [(16, 16), (8, 4), (32, 8), (64, 8), (6, 1), (32, 2), (3, 1), (20, 1), (48, 2),
                                        (33, 1)])

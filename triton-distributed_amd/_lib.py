@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libflash_decode_gfx950.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-FD_ABI_VERSION = 1
+FD_ABI_VERSION = 2
 
 # fd_dtype
 FD_F32, FD_F16, FD_BF16, FD_FP8_E4M3 = 0, 1, 2, 3
@@ -56,6 +56,7 @@ class FdParams(Structure):
         ("split_adapt", c_int32),
         ("max_kv_len", c_int32),
         ("seq_order_items", c_int32),
+        ("v_head_dim", c_int32),
     ]
 
 

@@ -32,6 +32,9 @@ int dtype_size(int dt) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Head dim of the V cache, of the partials and of the output.
+int v_dim(const fd_params* p) { return p->v_head_dim > 0 ? p->v_head_dim : p->head_dim; }
+
 // Magic number for n / d, exact for 0 <= n < 2^31: with l = ceil(log2 d) and k = 31 + l,
 // M = floor(2^k / d) + 1 fits in 32 bits and floor(n * M / 2^k) == floor(n / d).
 void div_magic(uint32_t d, uint32_t* magic, uint32_t* shift) {
@@ -232,6 +235,10 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     return fail(FD_ERR_TOO_LARGE, "%s: block table capacity exceeds 2^31 tokens", fn);
   const int D = p->head_dim;
   if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "%s: head_dim %d (64/128/256)", fn, D);
+  const int Dv = v_dim(p);
+  if (Dv != 64 && Dv != 128 && Dv != 256) return fail(FD_ERR_UNSUPPORTED, "%s: v_head_dim %d (64/128/256)", fn, Dv);
+  if (Dv != D && p->kv_dtype == FD_FP8_E4M3)
+    return fail(FD_ERR_UNSUPPORTED, "%s: an fp8 cache needs equal K and V head dims (%d, %d)", fn, D, Dv);
   const int qsz = dtype_size(p->q_dtype), kvsz = dtype_size(p->kv_dtype), msz = dtype_size(p->mid_dtype);
   if (!qsz || p->q_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: q_dtype %d", fn, p->q_dtype);
   if (!kvsz) return fail(FD_ERR_UNSUPPORTED, "%s: kv_dtype %d", fn, p->kv_dtype);
@@ -282,20 +289,20 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   // 204 -> 192 us; 4 MB of partials: no gain, so the plain store stays for those).
   {
     static const int forced = env_int("FD_STORE_THROUGH");   // tuning override for experiments: 1 always, 2 never
-    const int64_t partial_bytes = (int64_t)batch * p->q_heads * p->num_splits * D * msz;
+    const int64_t partial_bytes = (int64_t)batch * p->q_heads * p->num_splits * Dv * msz;
     a.store_through = a.vec_out && forced != 2 && (forced == 1 || partial_bytes >= kStoreThroughBytes) ? 1 : 0;
   }
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
   const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
-  const bool mfma_ok = mfma_shape_ok(D, p->kv_dtype) && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
+  const bool mfma_ok = mfma_shape_ok(D, p->kv_dtype) && Dv == D && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
                        aligned16(q) && stride_q_bs % 8 == 0 && stride_q_h % 8 == 0;
   bool use_mfma = mfma_ok;
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
-                "%s: MFMA path needs a 16-bit query with a KV cache of the same dtype or fp8-e4m3, and 16-byte aligned "
-                "q rows", fn);
+                "%s: MFMA path needs a 16-bit query with a KV cache of the same dtype or fp8-e4m3, equal K and V head "
+                "dims and 16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
@@ -407,7 +414,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   } else if (use_mfma) {
     rc = fd_launch_split_mfma((hipStream_t)stream, a, p->kv_dtype, waves, a.soft_cap > 0.f);
   } else {
-    rc = fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, waves);
+    rc = fd_launch_split_valu((hipStream_t)stream, a, p->kv_dtype, D, Dv, waves);
   }
   if (rc == FD_ERR_LAUNCH) return fail(rc, "%s: launch failed: %s", fn, hipGetErrorString(hipGetLastError()));
   if (rc != FD_OK) return fail(rc, "%s: no kernel for kv_dtype %d, head_dim %d, group %d", fn, p->kv_dtype, D, G);
@@ -516,19 +523,19 @@ int fd_decode_noalloc(void* stream, const void* q, const void* k_cache, const vo
                      nullptr, p);
   // fp32 partials [batch, Hq, S, D] followed by their fp32 LSEs [batch, Hq, S]
   const int64_t rows = (int64_t)batch * p->q_heads * p->num_splits;
-  const int64_t need = rows * (p->head_dim + 1) * 4;
+  const int64_t need = rows * (v_dim(p) + 1) * 4;
   if (need > (int64_t)FD_NOALLOC_SCRATCH_BYTES)
     return fail(FD_ERR_TOO_LARGE,
                 "%s: batch %d x q_heads %d x num_splits %d x (head_dim %d + 1) fp32 partials = %lld bytes exceed the "
                 "static workspace of %lld bytes; use fewer splits (fd_plan_splits) or fd_decode with a workspace of "
-                "your own", fn, batch, p->q_heads, p->num_splits, p->head_dim, (long long)need,
+                "your own", fn, batch, p->q_heads, p->num_splits, v_dim(p), (long long)need,
                 (long long)FD_NOALLOC_SCRATCH_BYTES);
   if (batch == 0) return FD_OK;
   void* ws = scratch_on_current_device(fn);
   if (!ws) return FD_ERR_LAUNCH;
   fd_params own = *p;
   own.mid_dtype = FD_F32;
-  const int64_t D = p->head_dim, S = p->num_splits;
+  const int64_t D = v_dim(p), S = p->num_splits;
   float* lse_split = (float*)ws + rows * D;
   return fd_decode(stream, q, k_cache, v_cache, ws, lse_split, out, lse_out, sm_scale, block_table, kv_lens, batch,
                    stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h,
@@ -544,7 +551,7 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
       p->page_size <= 0 || p->max_pages_per_seq <= 0)
     return fail(FD_ERR_INVALID_ARG, "%s: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0", fn);
   const int G = p->q_heads / p->kv_heads;
-  const bool mfma = mfma_shape_ok(p->head_dim, p->kv_dtype) && p->path != FD_PATH_VALU;
+  const bool mfma = mfma_shape_ok(p->head_dim, p->kv_dtype) && v_dim(p) == p->head_dim && p->path != FD_PATH_VALU;
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
   // fp8 rows of head_dim 64: two KV heads per wave (the usual cache layout has their rows side by side)
@@ -617,8 +624,8 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
     return fail(FD_ERR_INVALID_ARG, "fd_combine: mode %d", mode);
   if (num_extra > 0 && (!extra_out || !extra_lse))
     return fail(FD_ERR_INVALID_ARG, "fd_combine: num_extra > 0 needs extra_out and extra_lse");
-  if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)
-    return fail(FD_ERR_UNSUPPORTED, "fd_combine: head_dim %d (64/128/256)", p->head_dim);
+  if (v_dim(p) != 64 && v_dim(p) != 128 && v_dim(p) != 256)
+    return fail(FD_ERR_UNSUPPORTED, "fd_combine: head dim of the partials %d (64/128/256)", v_dim(p));
   if (!dtype_size(p->mid_dtype) || p->mid_dtype == FD_FP8_E4M3 || !dtype_size(p->out_dtype) ||
       p->out_dtype == FD_FP8_E4M3)
     return fail(FD_ERR_UNSUPPORTED, "fd_combine: mid_dtype %d / out_dtype %d", p->mid_dtype, p->out_dtype);
@@ -628,7 +635,7 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   a.mid_o = mid_o; a.mid_lse = mid_lse; a.out = out; a.lse_out = lse_out; a.seqlens = seqlens;
   a.extra_out = extra_out; a.extra_lse = extra_lse;
   a.s_mb = stride_mid_ob; a.s_mh = stride_mid_oh; a.s_ms = stride_mid_os; a.s_ob = stride_obs; a.s_oh = stride_oh;
-  a.batch = batch; a.Hq = q_heads; a.D = p->head_dim; a.num_partials = num_partials; a.num_extra = num_extra;
+  a.batch = batch; a.Hq = q_heads; a.D = v_dim(p); a.num_partials = num_partials; a.num_extra = num_extra;
   a.mode = mode; a.mid_dtype = p->mid_dtype; a.out_dtype = p->out_dtype;
   // rows that start on a multiple of four elements are read four values at a time
   a.vec_mid = ((reinterpret_cast<uintptr_t>(mid_o) & (4u * dtype_size(p->mid_dtype) - 1)) == 0 && stride_mid_ob % 4 == 0 &&
@@ -684,6 +691,7 @@ int fd_kv_append(void* stream, const void* k_new, const void* v_new, void* k_cac
   if (!append && !with_q) return fail(FD_ERR_INVALID_ARG, "%s: nothing to do (no k_new / v_new and no prep->q)", fn);
   const int D = p->head_dim;
   if (D != 64 && D != 128 && D != 256) return fail(FD_ERR_UNSUPPORTED, "%s: head_dim %d (64/128/256)", fn, D);
+  if (v_dim(p) != D) return fail(FD_ERR_UNSUPPORTED, "%s: K and V head dims must be equal (%d, %d)", fn, D, v_dim(p));
   const int ssz = dtype_size(p->q_dtype);
   if (!ssz || p->q_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: q_dtype %d", fn, p->q_dtype);
   const int src16 = 16 / ssz;

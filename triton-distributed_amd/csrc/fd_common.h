@@ -737,7 +737,7 @@ int fd_launch_split_mfma_fp8_d256(hipStream_t stream, const SplitArgs& a, int q_
 int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap);
 int fd_launch_split_mfma_fp8_d64(hipStream_t stream, const SplitArgs& a, int q_dtype, int waves, bool soft_cap,
                                  int kv_heads_per_wave);
-int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int waves);
+int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int v_head_dim, int waves);
 int fd_launch_combine(hipStream_t stream, const CombineArgs& a);
 int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, int32_t* order);
 int fd_launch_schedule_items(hipStream_t stream, const int32_t* kv_lens, int batch, int64_t capacity,

@@ -14,6 +14,11 @@
 // the tokens it sees (tokens rg, rg+TPI, ... of every tile) for up to GH query
 // heads; lane groups are merged with bpermutes at the end of the split, waves
 // of a workgroup through LDS.
+//
+// K and V head dims may differ (flash_decode.py:765-774 takes v_head_dim from the V cache, K_DIM / V_DIM :162-163):
+// a V row then has its own geometry -- LPRV lanes per row, TPIV rows per load instruction -- so the token a lane
+// group multiplies with V is not the token it scored; the probabilities move between the two geometries with
+// bpermutes, and the running maximum is kept wave-wide so that one rescale factor serves both.
 #include "fd_common.h"
 
 namespace {
@@ -68,17 +73,22 @@ struct KvTraits<FD_FP8_E4M3> {
   }
 };
 
-template <int KV, int D, int GH>
+template <int KV, int D, int DV, int GH>
 __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   using Tr = KvTraits<KV>;
   constexpr int E = Tr::E;            // elements per 16-byte chunk
-  constexpr int LPR = D / E;          // lanes per cache row
-  constexpr int TPI = 64 / LPR;       // rows per load instruction
-  constexpr int U = 4;                // load instructions per tile
+  constexpr int LPR = D / E;          // lanes per K row
+  constexpr int TPI = 64 / LPR;       // K rows per load instruction
+  constexpr int U = 4;                // K load instructions per tile
   constexpr int TILE = U * TPI;       // tokens per tile
+  constexpr int LPRV = DV / E;        // the same for V rows of DV elements
+  constexpr int TPIV = 64 / LPRV;
+  constexpr int UV = TILE / TPIV;
   constexpr int ESZ = 16 / E;         // bytes per element
-  constexpr int PART = (GH * D + 2 * GH + 3) & ~3;  // floats per wave partial (16-byte multiple)
+  constexpr int PART = (GH * DV + 2 * GH + 3) & ~3;  // floats per wave partial (16-byte multiple)
+  constexpr bool SAME = D == DV;
   static_assert(LPR >= 1 && LPR <= 64 && TILE <= 64, "unsupported geometry");
+  static_assert(LPRV >= 1 && LPRV <= 64 && UV >= 1 && UV * TPIV == TILE, "unsupported V geometry");
 
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
@@ -86,6 +96,8 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   const int wave = tid >> 6;
   const int rg = lane / LPR;          // lane group = row within a load instruction
   const int c = lane % LPR;           // chunk of the row
+  const int rgv = lane / LPRV;        // the same in the geometry of the V rows
+  const int cv = lane % LPRV;
 
   const WorkItem w = decode_work_item(a);   // this wave: KV head w.kvh, token sub-range w.sub of w.nsub
   if (w.skip) return;   // empty range, and the combine does not expect a partial from it
@@ -115,7 +127,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
 
   const int32_t* bt_row = a.bt + (int64_t)w.b * a.sbt;
   const char* kbase = (const char*)a.k + ((int64_t)w.kvh * a.sk_h) * ESZ + c * 16;
-  const char* vbase = (const char*)a.v + ((int64_t)w.kvh * a.sv_h) * ESZ + c * 16;
+  const char* vbase = (const char*)a.v + ((int64_t)w.kvh * a.sv_h) * ESZ + cv * 16;
   const int k_pitch = (int)(a.sk_t * ESZ);
   const int v_pitch = (int)(a.sv_t * ESZ);
 
@@ -134,14 +146,21 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
     for (int e = 0; e < E; ++e) acc[h][e] = 0.f;
   }
 
-  u32x4 kraw[U], vraw[U];
+  u32x4 kraw[U], vraw[UV];
   int rv_next = 0;
   auto issue = [&](int rv) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = __shfl(rv, u * TPI + rg);
       kraw[u] = load_stream_b128(kbase + (int64_t)row * k_pitch);
-      vraw[u] = load_stream_b128(vbase + (int64_t)row * v_pitch);
+      if constexpr (SAME) vraw[u] = load_stream_b128(vbase + (int64_t)row * v_pitch);
+    }
+    if constexpr (!SAME) {
+#pragma unroll
+      for (int u = 0; u < UV; ++u) {
+        const int row = __shfl(rv, u * TPIV + rgv);
+        vraw[u] = load_stream_b128(vbase + (int64_t)row * v_pitch);
+      }
     }
   };
   if (t0 < t1) {
@@ -150,12 +169,11 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   }
 
   for (int t = t0; t < t1; ++t) {
-    u32x4 kc[U], vc[U];
+    u32x4 kc[U], vc[UV];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      kc[u] = kraw[u];
-      vc[u] = vraw[u];
-    }
+    for (int u = 0; u < U; ++u) kc[u] = kraw[u];
+#pragma unroll
+    for (int u = 0; u < UV; ++u) vc[u] = vraw[u];
     if (t + 1 < t1) {
       issue(rv_next);
       if (t + 2 < t1) rv_next = tile_rows(t + 2);
@@ -183,6 +201,10 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
       float mx = sc[h][0];
 #pragma unroll
       for (int u = 1; u < U; ++u) mx = fmaxf(mx, sc[h][u]);
+      if (!SAME) {   // one maximum for the whole wave: the accumulators live in another lane geometry
+#pragma unroll
+        for (int o = LPR; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      }
       const float m_new = fmaxf(m[h], mx);
       // A lane group can see only masked tokens in the last tile: keep its state empty.
       const float m_use = m_new > -INFINITY ? m_new : 0.f;
@@ -198,24 +220,56 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
       for (int e = 0; e < E; ++e) acc[h][e] *= alpha;
       m[h] = m_new;
     }
+    if constexpr (SAME) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      float vf[E];
-      Tr::cvt(vc[u], vf);
+      for (int u = 0; u < U; ++u) {
+        float vf[E];
+        Tr::cvt(vc[u], vf);
 #pragma unroll
-      for (int h = 0; h < GH; ++h)
+        for (int h = 0; h < GH; ++h)
 #pragma unroll
-        for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p[h][u], vf[e], acc[h][e]);
+          for (int e = 0; e < E; ++e) acc[h][e] = fmaf(p[h][u], vf[e], acc[h][e]);
+      }
+    } else {
+      // V load uv holds, for this lane, token uv * TPIV + rgv of the tile; its probability sits in the K geometry
+      // at load u = token / TPI, lane group token % TPI (any lane of that group).
+#pragma unroll
+      for (int uv = 0; uv < UV; ++uv) {
+        float vf[E];
+        Tr::cvt(vc[uv], vf);
+#pragma unroll
+        for (int h = 0; h < GH; ++h) {
+          float pv;
+          if constexpr (TPIV >= TPI) {
+            constexpr int R = TPIV / TPI;        // K loads that one V load spans
+            const int src = (rgv % TPI) * LPR;
+            pv = 0.f;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+              const float cand = __shfl(p[h][uv * R + j], src);
+              pv = (rgv / TPI == j) ? cand : pv;
+            }
+          } else {
+            constexpr int R = TPI / TPIV;        // V loads that one K load spans
+            pv = __shfl(p[h][uv / R], ((uv % R) * TPIV + rgv) * LPR);
+          }
+#pragma unroll
+          for (int e = 0; e < E; ++e) acc[h][e] = fmaf(pv, vf[e], acc[h][e]);
+        }
+      }
     }
   }
 
-  // ---- merge the TPI lane groups of the wave (all-reduce over lanes with equal c)
+  // ---- merge the lane groups of the wave (all-reduce over lanes with equal chunk index)
 #pragma unroll
   for (int h = 0; h < GH; ++h) {
     float M = m[h];
+    float sf = 1.0f;
+    if (SAME) {   // every lane group kept its own running maximum
 #pragma unroll
-    for (int o = LPR; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
-    const float sf = M > -INFINITY ? fd_exp2(m[h] - M) : 0.f;
+      for (int o = LPR; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
+      sf = M > -INFINITY ? fd_exp2(m[h] - M) : 0.f;
+    }
     float L = l[h] * sf;
 #pragma unroll
     for (int o = LPR; o < 64; o <<= 1) L += __shfl_xor(L, o);
@@ -223,41 +277,41 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
     for (int e = 0; e < E; ++e) {
       float x = acc[h][e] * sf;
 #pragma unroll
-      for (int o = LPR; o < 64; o <<= 1) x += __shfl_xor(x, o);
+      for (int o = LPRV; o < 64; o <<= 1) x += __shfl_xor(x, o);
       acc[h][e] = x;
     }
     m[h] = M;
     l[h] = L;
   }
   float* part = (float*)smem + wave * PART;
-  if (rg == 0) {
+  if (rgv == 0) {
     const float v_scale = KV == FD_FP8_E4M3 ? a.v_scale[w.kvh] : 1.0f;   // V dequantisation, once
 #pragma unroll
     for (int h = 0; h < GH; ++h) {
 #pragma unroll
-      for (int e = 0; e < E; ++e) part[h * D + c * E + e] = acc[h][e] * v_scale;
-      if (c == 0) {
-        part[GH * D + h] = m[h];
-        part[GH * D + GH + h] = l[h];
+      for (int e = 0; e < E; ++e) part[h * DV + cv * E + e] = acc[h][e] * v_scale;
+      if (cv == 0) {
+        part[GH * DV + h] = m[h];
+        part[GH * DV + GH + h] = l[h];
       }
     }
   }
   __syncthreads();
-  cta_merge_store<GH, D>(a, (const float*)smem, PART, w, nheads);
-  if (a.tickets) fused_combine<D>(a, w, head0, nheads, (float*)smem);  // hpw == 1 when fused
+  cta_merge_store<GH, DV>(a, (const float*)smem, PART, w, nheads);
+  if (a.tickets) fused_combine<DV>(a, w, head0, nheads, (float*)smem);  // hpw == 1 when fused
 }
 
-template <int KV, int D>
-int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
+template <int KV, int D, int DV>
+int launch_kdv(hipStream_t stream, const SplitArgs& a, int waves) {
   const dim3 grid = fd_split_grid(a);
   const unsigned block = 64u * waves;
   void (*kern)(const SplitArgs) = nullptr;
   int gh = a.hbsz;
-  if (gh == 1) kern = fd_split_valu_kernel<KV, D, 1>;
-  else if (gh == 2) kern = fd_split_valu_kernel<KV, D, 2>;
-  else if (gh == 4) kern = fd_split_valu_kernel<KV, D, 4>;
+  if (gh == 1) kern = fd_split_valu_kernel<KV, D, DV, 1>;
+  else if (gh == 2) kern = fd_split_valu_kernel<KV, D, DV, 2>;
+  else if (gh == 4) kern = fd_split_valu_kernel<KV, D, DV, 4>;
   else return FD_ERR_UNSUPPORTED;
-  size_t lds = (size_t)waves * ((gh * D + 2 * gh + 3) & ~3) * 4;
+  size_t lds = (size_t)waves * ((gh * DV + 2 * gh + 3) & ~3) * 4;
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
     const size_t need = (size_t)(a.S + a.num_extra) * gh * 4;
     if (need > lds) lds = need;
@@ -271,24 +325,37 @@ int launch_kd(hipStream_t stream, const SplitArgs& a, int waves) {
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
 }
 
+template <int KV, int D>
+int launch_kd(hipStream_t stream, const SplitArgs& a, int v_head_dim, int waves) {
+  if (v_head_dim == D) return launch_kdv<KV, D, D>(stream, a, waves);
+  if constexpr (KV != FD_FP8_E4M3) {   // K and V head dims that differ: not for fp8 caches
+    switch (v_head_dim) {
+      case 64: return launch_kdv<KV, D, 64>(stream, a, waves);
+      case 128: return launch_kdv<KV, D, 128>(stream, a, waves);
+      case 256: return launch_kdv<KV, D, 256>(stream, a, waves);
+    }
+  }
+  return FD_ERR_UNSUPPORTED;
+}
+
 template <int KV>
-int launch_k(hipStream_t stream, const SplitArgs& a, int head_dim, int waves) {
+int launch_k(hipStream_t stream, const SplitArgs& a, int head_dim, int v_head_dim, int waves) {
   switch (head_dim) {
-    case 64: return launch_kd<KV, 64>(stream, a, waves);
-    case 128: return launch_kd<KV, 128>(stream, a, waves);
-    case 256: return launch_kd<KV, 256>(stream, a, waves);
+    case 64: return launch_kd<KV, 64>(stream, a, v_head_dim, waves);
+    case 128: return launch_kd<KV, 128>(stream, a, v_head_dim, waves);
+    case 256: return launch_kd<KV, 256>(stream, a, v_head_dim, waves);
     default: return FD_ERR_UNSUPPORTED;
   }
 }
 
 }  // namespace
 
-int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int waves) {
+int fd_launch_split_valu(hipStream_t stream, const SplitArgs& a, int kv_dtype, int head_dim, int v_head_dim, int waves) {
   switch (kv_dtype) {
-    case FD_F32: return launch_k<FD_F32>(stream, a, head_dim, waves);
-    case FD_F16: return launch_k<FD_F16>(stream, a, head_dim, waves);
-    case FD_BF16: return launch_k<FD_BF16>(stream, a, head_dim, waves);
-    case FD_FP8_E4M3: return launch_k<FD_FP8_E4M3>(stream, a, head_dim, waves);
+    case FD_F32: return launch_k<FD_F32>(stream, a, head_dim, v_head_dim, waves);
+    case FD_F16: return launch_k<FD_F16>(stream, a, head_dim, v_head_dim, waves);
+    case FD_BF16: return launch_k<FD_BF16>(stream, a, head_dim, v_head_dim, waves);
+    case FD_FP8_E4M3: return launch_k<FD_FP8_E4M3>(stream, a, head_dim, v_head_dim, waves);
     default: return FD_ERR_UNSUPPORTED;
   }
 }

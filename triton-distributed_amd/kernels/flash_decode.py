@@ -117,16 +117,19 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
 
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
                  waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0,
-                 max_kv_len=0) -> FdParams:
+                 max_kv_len=0, v_head_dim=0) -> FdParams:
     # the scalar fields are the same from step to step: filled once per combination, copied per call
+    v_head_dim = v_head_dim or q.shape[2]
     key = (q.shape, k_cache.shape, block_table.shape[1], q.dtype, k_cache.dtype, k_scale is not None, kv_split, soft_cap,
-           mid_dtype, out_dtype, path, waves_per_block, split_align, split_adapt, seq_order_items, max_kv_len)
+           mid_dtype, out_dtype, path, waves_per_block, split_align, split_adapt, seq_order_items, max_kv_len,
+           v_head_dim)
     template = _PARAMS_CACHE.get(key)
     if template is None:
         t = FdParams()
         t.q_heads = q.shape[1]
         t.kv_heads = k_cache.shape[2]
         t.head_dim = q.shape[2]
+        t.v_head_dim = v_head_dim if v_head_dim != q.shape[2] else 0
         t.page_size = k_cache.shape[1]
         t.num_splits = kv_split
         t.num_pages = k_cache.shape[0]
@@ -169,7 +172,7 @@ def _hint(max_kv_len, capacity):
 
 
 def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=None, path="auto", waves_per_block=0,
-                max_kv_len=None):
+                max_kv_len=None, v_head_dim=0):
     """The split plan of a decode step whose partials stay inside the library: ``(num_splits, split_adapt)`` --
     grid slots per sequence and the ranges every sequence gets however short it is (``fd_plan_splits``,
     ``fd_plan_min_splits``; cached by shape).  ``kv_split`` is the caller's bound, -1 leaves it to the library;
@@ -180,12 +183,12 @@ def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=N
     hint = _hint(max_kv_len, capacity)
     bound = auto_split_bound(hint or capacity) if kv_split == -1 else kv_split
     key = (batch, q_heads, kv_heads, q_head_dim, page_size, bound, block_table.shape[1], k_cache.dtype,
-           k_scale is not None, path, hint)
+           k_scale is not None, path, hint, v_head_dim or q_head_dim)
     planned = _PLAN_CACHE.get(key)
     if planned is None:
         lib = load_library()
         plan = _make_params(q, k_cache, block_table, bound, 0.0, FD_F32, FD_F32, k_scale, v_scale, path,
-                            waves_per_block, max_kv_len=hint)
+                            waves_per_block, max_kv_len=hint, v_head_dim=v_head_dim)
         planned = (lib.fd_plan_splits(byref(plan), batch), lib.fd_plan_min_splits(byref(plan), batch))
         if min(planned) < 0:
             check(min(planned))
@@ -207,7 +210,6 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
     v_head_dim = v_cache.shape[-1]
     assert q_heads % kv_heads == 0
-    assert v_head_dim == k_head_dim, "the gfx950 kernels need equal K and V head dims"
     _require_cuda(q, k_cache, v_cache, kv_lens, block_table, output_split, output_combine)
     assert kv_lens.dtype == torch.int32 and block_table.dtype == torch.int32
     q_st, k_st, v_st = q.stride(), k_cache.stride(), v_cache.stride()
@@ -229,7 +231,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             # may get more than the reference's 32).  The grid has num_splits slots per sequence; a sequence uses as
             # many as its own length asks for.
             num_splits, split_adapt = plan_decode(q, k_cache, block_table, kv_split, k_scale=k_scale, v_scale=v_scale,
-                                                  path=path, waves_per_block=waves_per_block, max_kv_len=max_kv_len)
+                                                  path=path, waves_per_block=waves_per_block, max_kv_len=max_kv_len,
+                                                  v_head_dim=v_head_dim)
         n_o = batch * q_heads * num_splits * v_head_dim
         n_l = batch * q_heads * num_splits
         direct = (num_splits == 1 and extra_partials is None and not fuse_combine
@@ -284,7 +287,7 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
                      v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
-                     split_adapt, 0, _hint(max_kv_len, block_table.shape[1] * page_size))
+                     split_adapt, 0, _hint(max_kv_len, block_table.shape[1] * page_size), v_head_dim)
     if want_items:
         if item_order is None:
             item_order = item_order_buffer(batch, num_splits, q.device)

@@ -23,7 +23,7 @@ class FdParams(Structure):            # struct fd_params, include/flash_decode.h
                 ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
                 ("path", c_int32), ("waves_per_block", c_int32), ("seq_order_lens", c_void_p),
                 ("split_align", c_int32), ("split_adapt", c_int32),
-                ("max_kv_len", c_int32), ("seq_order_items", c_int32)]
+                ("max_kv_len", c_int32), ("seq_order_items", c_int32), ("v_head_dim", c_int32)]
 
 _lib = ctypes.CDLL(os.environ.get("FD_LIBRARY_PATH") or
                    os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflash_decode_gfx950.so"))
