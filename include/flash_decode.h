@@ -103,7 +103,7 @@ typedef struct fd_params {
                                empty).  The result of a step is the same; the partials are not
                                the reference's.  fd_combine applies the same rule.          */
   int32_t split_adapt;      /* 0: every sequence is cut into num_splits ranges (the reference).
-                               k > 0 (a power of two; needs split_align > 0): a range of a sequence
+                               k > 0 (a power of two; needs split_align > 0; num_splits may be any count): a range of a sequence
                                of n tokens holds max(ceil(n / num_splits), min(ceil(n / k), w))
                                tokens, w = ceil(n / 8) kept within [1024, 4096] -- at least k
                                ranges; beyond that 1024-token ranges up to 8 of them, 8 ranges up
@@ -286,10 +286,13 @@ FD_API int fd_schedule_items(void* stream, const int32_t* kv_lens, int32_t batch
  * not look at.  NUM_KV_SPLITS is a tuning constant in the reference (flash_decode.py:779:
  * 32 unless the caller says otherwise); the result of a step does not depend on it.  When
  * the partial workspace is internal, fewer and longer splits mean fewer workgroup
- * prologues and fewer partials for the combine.  Returns a power of two, at most
- * params->num_splits: the smallest split count that (1) gives one workgroup per CU (256) with
+ * prologues and fewer partials for the combine.  Returns a count of at most
+ * params->num_splits: the smallest power of two that (1) gives one workgroup per CU (256) with
  * the workgroup at its full width (sibling KV heads that share 512 bytes of a token row, or head
- * blocks of one KV head), raised (2) until the workgroups are a whole number per CU or at
+ * blocks of one KV head) -- or, where no power of two does because the heads do not divide the CU
+ * count (12 KV heads), the count just under one workgroup per CU (42 with sibling heads, 21 without
+ * them where a split would otherwise hold fewer than 512 tokens) --, raised (2) until the workgroups
+ * are a whole number per CU or at
  * least four per CU, as long as a split of a full-length sequence keeps 512 tokens, and (3) in
  * a batch until no split of a full-length sequence exceeds 4096 tokens or 32 splits are reached (VALU kernel: about
  * 2048 waves with four per split instead of (1) and (2)); or a negative fd_status.
@@ -302,7 +305,7 @@ FD_API int fd_plan_splits(const fd_params* params, int32_t batch);
  * The part of fd_plan_splits' count that the shape needs to fill the chip (its rules 1 and 2, or the VALU
  * rule), without the part that only bounds the length of a split in a batch: the value for
  * fd_params.split_adapt.  No counterpart in the reference (one split count for all sequences,
- * flash_decode.py:193-195).  Returns the count (a power of two >= 1, not clamped to params->num_splits) or a negative
+ * flash_decode.py:193-195).  Returns the count rounded up to a power of two (>= 1, not clamped to params->num_splits) or a negative
  * fd_status.
  */
 FD_API int fd_plan_min_splits(const fd_params* params, int32_t batch);

@@ -212,11 +212,15 @@ def test_split_plan_policy(fd):
     assert plan(64, 40, 2, 32, 256, kv=L.FD_FP8_E4M3, D=64) == 2
     assert plan(8, 8, 8, 32, 512, kv=L.FD_F32) == 8  # VALU path (fp32 cache): 2048 waves with 4 waves per (head, split)
     assert plan(2, 8, 8, 32, 512) == 32
-    assert plan(3, 32, 8, 32, 512) == 32           # 21.3 -> the next power of two
-    assert plan(3, 32, 8, 24, 512) == 16           # ... and down again when the caller allows fewer
-    assert plan(1, 96, 12, 128, 65536, P=1) == 128  # 12 KV heads: 64 splits would be 1.5 workgroups per CU, 128 are 3
+    # groups that do not divide the CU count: the count just under one workgroup per CU, without sibling heads
+    # where a split would otherwise hold fewer than 512 tokens
+    assert plan(3, 32, 8, 32, 512) == 10           # 24 groups x 10 = 240 workgroups
+    assert plan(3, 32, 8, 8, 512) == 8             # ... or what the caller allows
+    assert plan(1, 96, 12, 128, 65536, P=1) == 42  # 12 KV heads: 12 x 42 / 2 sibling heads = 252 workgroups
+    assert plan(1, 96, 12, 128, 16384, P=1) == 21  # short splits: 12 x 21 = 252 workgroups of one head
+    assert plan(1, 96, 12, 32, 65536, P=1) == 32   # the caller's bound wins
     assert plan(1, 8, 1, 256, 65536) == 256        # one KV head: one split per CU
-    assert plan(1, 96, 12, 128, 1 << 20, P=1) == 128
+    assert plan(1, 96, 12, 128, 1 << 20, P=1) == 42
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1
     # the part of the plan that fills the chip, without the bound on the length of a split: what a sequence gets
@@ -230,6 +234,7 @@ def test_split_plan_policy(fd):
     assert plan(8, 32, 8, 32, 8192) == 32                                      # ... while the grid covers the capacity
     assert fill(64, 32, 8, 32, 8192) == 1 and plan(64, 32, 8, 32, 8192) == 32  # a batch fills the chip by itself
     assert fill(1, 8, 1, 256, 65536) == 256
+    assert fill(1, 96, 12, 128, 65536, P=1) == 64   # split_adapt is a power of two: the next one above 42
     assert plan(64, 32, 8, 256, 65536) == 32       # a table for 1 M tokens: not more than 32 slots per sequence for balance
     assert plan(2, 32, 8, 256, 65536) == 32 and plan(1, 32, 8, 256, 65536) == 64
     assert fill(0, 32, 8, 32, 512) < 0 and lib.fd_plan_min_splits(None, 1) < 0

@@ -82,10 +82,8 @@ bool fp8_d64_pairs(int group, int kv_heads) { return group <= 16 && kv_heads % 2
 int check_split_adapt(const char* fn, const fd_params* p) {
   const int k = p->split_adapt;
   if (k == 0) return FD_OK;
-  if (k < 0 || (k & (k - 1)) || p->split_align <= 0 || (p->num_splits & (p->num_splits - 1)))
-    return fail(FD_ERR_INVALID_ARG,
-                "%s: split_adapt %d needs a power of two, split_align > 0 and a power-of-two num_splits (%d)", fn, k,
-                p->num_splits);
+  if (k < 0 || (k & (k - 1)) || p->split_align <= 0)
+    return fail(FD_ERR_INVALID_ARG, "%s: split_adapt %d needs a power of two and split_align > 0", fn, k);
   return FD_OK;
 }
 
@@ -128,7 +126,8 @@ bool env_no_chunk() {
 int choose_waves(int64_t head_splits, int64_t max_tokens_per_split, int tile, int64_t target, int max_waves) {
   int64_t tiles = (max_tokens_per_split + tile - 1) / tile;
   int w = 1;
-  while (w < max_waves && head_splits * w < target && w * 2 <= tiles) w *= 2;
+  // (a grid a few workgroups short of one per CU -- 252 -- counts as reaching the target)
+  while (w < max_waves && head_splits * w * 16 < target * 15 && w * 2 <= tiles) w *= 2;
   const int e = env_waves();
   if (e == 1 || e == 2 || e == 4 || e == 8) w = e;
   return w < max_waves ? w : max_waves;
@@ -140,7 +139,8 @@ int choose_heads_per_group(int kv_heads, int row_bytes, int waves, int64_t head_
   int h = row_bytes > 0 ? 512 / row_bytes : 1;
   if (env_heads() > 0) h = env_heads();
   if (h < 1) h = 1;
-  while (h > 1 && (kv_heads % h != 0 || h * waves > max_waves || head_splits / h < kMinWorkgroups)) h >>= 1;
+  // (a grid that misses one workgroup per CU by a few -- 12 KV heads x 42 splits / 2 = 252 -- still counts as full)
+  while (h > 1 && (kv_heads % h != 0 || h * waves > max_waves || head_splits / h < kMinWorkgroups * 15 / 16)) h >>= 1;
   // Between one and one and a half workgroups per CU the busiest CUs hold two workgroups of h members; with half the
   // members they hold three of h / 2 (measured 3 - 7 % faster there: B = 5 x 5000 tokens 22.4 -> 20.8 us)
   const int64_t nwg = head_splits / h;
@@ -573,6 +573,20 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
       while (members > 1 && kv_units % members != 0) members >>= 1;
     }
     while (s * groups < kMinWorkgroups * members) s <<= 1;
+    if (s * groups != kMinWorkgroups * members) {
+      // (1b) The groups do not divide the CU count (12 KV heads): no power of two gives one workgroup per CU.  The
+      // count just under it does -- 12 x 42 / 2 = 252 workgroups in one round -- with far fewer partials than the
+      // power of two that reaches a whole number per CU (128 splits, 768 workgroups): one query, 96 / 12 heads,
+      // 65536 tokens 72.2 -> 68.2 us, 1048576 tokens 953.6 -> 949.0 us.  Where a split would hold fewer than 512
+      // tokens the sibling members are given up for half as many splits (16384 tokens: 25.5 -> 23.3 us with 21).
+      int64_t m = members;
+      int64_t exact = kMinWorkgroups * m / groups;
+      while (m > 1 && exact > 0 && max_tokens / exact < 512) {
+        m >>= 1;
+        exact = kMinWorkgroups * m / groups;
+      }
+      if (exact >= 2 && exact * groups * 10 >= kMinWorkgroups * m * 9) return exact;
+    }
     // (2) ... and a whole number of workgroups per CU, or at least four, while a split of a full-length sequence
     // keeps 512 tokens: equal work items run in one round, and 1.5 workgroups per CU take as long as 2
     while (s < p->num_splits && (s * groups / members) % kMinWorkgroups != 0 &&
@@ -587,7 +601,10 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
 
 int fd_plan_min_splits(const fd_params* p, int32_t batch) {
   const int64_t s = plan_fill_splits("fd_plan_min_splits", p, batch);
-  return (int)(s > 65536 ? 65536 : s);
+  if (s < 0) return (int)s;
+  int64_t pow2 = 1;   // fd_params.split_adapt is a power of two: the next one
+  while (pow2 < s && pow2 < 65536) pow2 <<= 1;
+  return (int)pow2;
 }
 
 int fd_plan_splits(const fd_params* p, int32_t batch) {
@@ -602,9 +619,11 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   if (batch > 1) {
     while (s * kMaxTokensPerSplit < max_tokens && s < kMaxBalanceSplits) s <<= 1;
   }
-  // Powers of two throughout: with sequence lengths that are powers of two (or multiples of large ones) every split
-  // then starts on a tile boundary and the waves of a workgroup get equal runs.
-  while (s > p->num_splits) s >>= 1;
+  // Powers of two where the shape allows: with sequence lengths that are powers of two (or multiples of large ones)
+  // every split then starts on a tile boundary and the waves of a workgroup get equal runs.
+  const bool pow2 = (s & (s - 1)) == 0;
+  while (pow2 && s > p->num_splits) s >>= 1;
+  if (s > p->num_splits) s = p->num_splits;
   if (s < 1) s = 1;
   return (int)s;
 }
@@ -646,10 +665,8 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   a.per_mask = p->split_align ? p->split_align - 1 : 0;
   if (mode != FD_COMBINE_RANK) {
     a.adapt = p->split_adapt;
-    if (a.adapt < 0 || (a.adapt & (a.adapt - 1)) || (a.adapt > 0 && (p->split_align <= 0 || (num_partials & (num_partials - 1)))))
-      return fail(FD_ERR_INVALID_ARG,
-                  "fd_combine: split_adapt %d needs a power of two, split_align > 0 and a power-of-two num_partials (%d)",
-                  a.adapt, num_partials);
+    if (a.adapt < 0 || (a.adapt & (a.adapt - 1)) || (a.adapt > 0 && p->split_align <= 0))
+      return fail(FD_ERR_INVALID_ARG, "fd_combine: split_adapt %d needs a power of two and split_align > 0", a.adapt);
   }
   div_magic((uint32_t)num_partials, &a.s_magic, &a.s_shift);
   // Lengths beyond the block table's capacity are clamped exactly as the split kernels clamp them, so that both
