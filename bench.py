@@ -44,6 +44,7 @@ def parse_args():
                     help="override the workload's kv_split (experiments); -1: the library's own choice")
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-targets", action="store_true",
                     help="skip the other north-star figures (exact split counts, configs 3, 4, 5) that the default "
@@ -351,6 +352,23 @@ def main():
     ms_per_step = max(gpu_ms, 0.0) / args.steps
     us_per_step = ms_per_step * 1e3
 
+    # ---- the same step replayed from a HIP graph (a serving loop captures its step): 8 steps per graph, rotating
+    # over the pools like the eager loop
+    graph_us = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(8):
+                step(i)
+        graph_us = _time_us(torch, lambda _: graph.replay(), max(5, args.steps // 4), 3) / 8
+        del graph
+
     # ---- dominant kernel alone (split-KV), HIP events on the launch stream
     from ctypes import byref
     lib = fd.load_library()
@@ -453,6 +471,7 @@ def main():
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        "hip_graph_replay_us_per_step": None if graph_us is None else round(graph_us, 3),
         "clock_ramp_ms": round(ramp_ms),
         "roofline": {"bound": "hbm", "kernel": "fd_split_*_kernel (split-KV decode)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
