@@ -166,21 +166,24 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   }
 }
 
-// Up to MAXP (16 or 32) partials produced by this library's split kernel in the same call, rows readable four values at a time,
-// LSEs in their own fp32 buffer: every slot is written (an empty split holds out = 0, lse = -inf), so validity needs
-// no kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which leaves one dependent
-// memory round trip.  The kernel is short on purpose: one workgroup per output row on a chip that the step's split
-// kernel has just vacated runs at one wave per SIMD, where every instruction of the wave is latency.  Thread (r, c):
-// partials r, r + ROWS, ... and 128-bit column chunk c.  Every thread reads all LSEs of the row itself (the same few
-// cache lines for the whole workgroup) for the maximum, so nothing goes through LDS before the final sum.
-template <int D, int MAXP>
+// Up to MAXP (16, 32 or 64) partials produced by this library's split kernel in the same call, rows readable four
+// values at a time, LSEs in their own fp32 buffer: every slot is written (an empty split holds out = 0, lse = -inf),
+// so validity needs no kv_lens, and the row loads do not wait for the LSEs -- both are requested at once, which
+// leaves one dependent memory round trip.  The kernel is short on purpose: one workgroup per output row on a chip
+// that the step's split kernel has just vacated runs at one wave per SIMD, where every instruction of the wave is
+// latency.  Thread (r, c): partials r, r + ROWS, ... and 128-bit column chunk c.  Lane i of every wave loads LSE i
+// (MAXP <= 64 = one per lane); the maximum is a butterfly over the wave and a thread takes the LSEs of its own
+// partials from the lanes that hold them, so nothing goes through LDS before the final sum.
+template <int D, int MAXP, int MID>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const CombineArgs a) {
   constexpr int CG = D / 4;
   constexpr int ROWS = kCombineThreads / CG;
   constexpr int PASSES = (MAXP + ROWS - 1) / ROWS;
+  static_assert(MAXP <= 64, "one LSE per lane");
   __shared__ __align__(16) float s_acc[ROWS][D];
   __shared__ float s_l[ROWS];
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
   const int b = blockIdx.x / a.Hq;
   const int h = blockIdx.x - b * a.Hq;
   const int S = a.num_partials;
@@ -189,19 +192,17 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
   const int r = tid / CG;
   const int c = tid - r * CG;
   f32x4 o[PASSES];
-  float own[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int s = r + p * ROWS;
     o[p] = f32x4{0.f, 0.f, 0.f, 0.f};
-    own[p] = -INFINITY;
     if (s < S) {
       const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
-      if (a.mid_dtype == FD_F32) {
+      if constexpr (MID == FD_F32) {
         o[p] = *(const f32x4*)((const float*)a.mid_o + off);
       } else {
         const u32x2 w = *(const u32x2*)((const uint16_t*)a.mid_o + off);
-        if (a.mid_dtype == FD_F16) {
+        if constexpr (MID == FD_F16) {
           o[p] = f32x4{f16_bits_to_f32(w[0] & 0xffffu), f16_bits_to_f32(w[0] >> 16), f16_bits_to_f32(w[1] & 0xffffu),
                        f16_bits_to_f32(w[1] >> 16)};
         } else {
@@ -209,30 +210,21 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
                        bf16_bits_to_f32(w[1] >> 16)};
         }
       }
-      own[p] = lse_row[s];
     }
   }
-  float M = -INFINITY;
-  if ((S & 3) == 0) {   // the row of LSEs is 16-byte aligned
+  const float mine = lane < S ? lse_row[lane] : -INFINITY;   // LSE of partial `lane`
+  float M = mine;
 #pragma unroll
-    for (int q = 0; q < MAXP / 4; ++q) {
-      if (4 * q < S) {
-        const f32x4 v = *(const f32x4*)(lse_row + 4 * q);
-        M = fmaxf(fmaxf(M, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
-      }
-    }
-  } else {
-    for (int q = 0; q < S; ++q) M = fmaxf(M, lse_row[q]);
-  }
+  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
   float L = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  if (M > -INFINITY) {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const float wgt = __expf(own[p] - M);   // exp(-inf) = 0 for empty / absent splits
-      acc += o[p] * wgt;
-      L += wgt;
-    }
+  for (int p = 0; p < PASSES; ++p) {
+    const int s = r + p * ROWS;
+    const float own = __shfl(mine, s & 63);          // -inf for empty and absent splits: weight 0
+    const float wgt = M > -INFINITY && s < S ? __expf(own - M) : 0.f;
+    acc += o[p] * wgt;
+    L += wgt;
   }
   *(f32x4*)&s_acc[r][4 * c] = acc;
   if (c == 0) s_l[r] = L;
@@ -301,12 +293,12 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   CombineArgs a = args;
   const int64_t rows = (int64_t)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
-  // the short kernel: this library's own partials in the same call, all slots written, at most 32 of them (with 64 a
-  // thread would hold 8 rows and 64 LSEs, and the registers for that cost the occupancy that large batches need:
-  // config 5's shape with 64 splits 24.7 us against 13 us in the general kernel)
-  const int np_own = a.num_partials <= 16 ? 16 : 32;
-  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 && a.num_partials <= 32 &&
-                     a.vec_mid && a.mid_lse && (reinterpret_cast<uintptr_t>(a.mid_lse) & 15u) == 0;
+  // the short kernel: this library's own partials in the same call, all slots written, at most 64 of them -- above
+  // 32 only where there is a workgroup per CU: with few output rows (one long sequence: 96 rows x 42 partials) the
+  // general kernel, which spreads a row over several workgroups, is the faster one (5.0 against 5.7 us)
+  const int np_own = a.num_partials <= 16 ? 16 : (a.num_partials <= 32 ? 32 : 64);
+  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 && a.vec_mid && a.mid_lse &&
+                     (a.num_partials <= 32 || (a.num_partials <= 64 && rows >= 256));
   // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
   // one workgroup per CU and a thread would still have more than two partials to walk.
   int cg = a.D / 4;
@@ -317,13 +309,15 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   const int64_t wgs = small ? rows : rows * (a.D / 4 / cg);
   if (wgs >= ((int64_t)1 << 31)) return FD_ERR_TOO_LARGE;
   const unsigned grid = (unsigned)wgs;
-#define FD_OWN(D_) (np_own == 16 ? fd_combine_own_kernel<D_, 16> : fd_combine_own_kernel<D_, 32>)
+#define FD_OWN_P(D_, M_) (np_own == 16 ? fd_combine_own_kernel<D_, 16, M_> : np_own == 32 ? fd_combine_own_kernel<D_, 32, M_> : fd_combine_own_kernel<D_, 64, M_>)
+#define FD_OWN(D_) (a.mid_dtype == FD_F32 ? FD_OWN_P(D_, FD_F32) : a.mid_dtype == FD_F16 ? FD_OWN_P(D_, FD_F16) : FD_OWN_P(D_, FD_BF16))
   switch (a.D) {
     case 64: kern = small ? FD_OWN(64) : fd_combine_kernel<64>; break;
     case 128: kern = small ? FD_OWN(128) : fd_combine_kernel<128>; break;
     case 256: kern = small ? FD_OWN(256) : fd_combine_kernel<256>; break;
     default: return FD_ERR_UNSUPPORTED;
   }
+#undef FD_OWN_P
 #undef FD_OWN
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;
