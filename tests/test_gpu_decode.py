@@ -497,6 +497,57 @@ def test_output_split_layout(fd, mid_dtype, num_heads):
     assert_out_close(outc, ref)
 
 
+# ---- exactly the caller's splits on the chunked path (one workgroup walks consecutive splits, every wave stores one
+# partial per split): every partial against the per-split model (flash_decode.py:193-239), odd split counts that the
+# chunk does not divide, sequences shorter than the split count, empty ones, two head blocks per wave, fp8
+@pytest.mark.parametrize("kind", ["bf16", "fp16_g32", "fp8", "bf16_mha"])
+@pytest.mark.parametrize("S,mid_dtype", [(32, torch.float32), (24, torch.bfloat16), (7, torch.float16), (64, torch.float32),
+                                         (3, torch.float32)])
+@pytest.mark.parametrize("soft_cap", [0, 30])
+def test_exact_splits_on_chunked_work_items(fd, kind, S, mid_dtype, soft_cap):
+    Hq, Hkv, dtype, fp8 = {"bf16": (32, 8, torch.bfloat16, False), "fp16_g32": (128, 4, torch.float16, False),
+                           "fp8": (64, 8, torch.bfloat16, True), "bf16_mha": (8, 8, torch.bfloat16, False)}[kind]
+    lens = [4099, 18, 0, 1, 2049, 777, 64, 33]
+    wl = fd.utils.make_paged_workload("chunked_" + kind, lens, Hq, Hkv, 128, 16, dtype, S, seed=61 + S,
+                                      soft_cap=float(soft_cap), fp8_kv=fp8)
+    # the launch must actually be chunked for this to test anything: the library's own plan has fewer splits
+    L = fd._lib
+    from ctypes import byref
+    p = L.FdParams()
+    p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits = Hq, Hkv, 128, 16, S
+    p.num_pages, p.max_pages_per_seq = wl.k_cache.shape[0], wl.block_table.shape[1]
+    p.q_dtype, p.kv_dtype = L.fd_dtype_of(wl.q), (L.FD_FP8_E4M3 if fp8 else L.fd_dtype_of(wl.k_cache))
+    planned = fd.load_library().fd_plan_splits(byref(p), len(lens))
+    g = wl.to(DEV)
+    B, D = len(lens), 128
+    mid = torch.full((B, Hq, S, D + 1), float("nan"), dtype=mid_dtype, device=DEV)
+    out, lse = run_decode(fd, wl, output_split=mid)
+    kc, vc = wl.k_cache, wl.v_cache
+    if fp8:
+        kc = oracle.dequant_fp8_cache(kc.view(torch.uint8), wl.k_scale)
+        vc = oracle.dequant_fp8_cache(vc.view(torch.uint8), wl.v_scale)
+    model = oracle.model_split_kv(wl.q.float(), kc.float(), vc.float(), lens, wl.block_table, wl.scale, S,
+                                  soft_cap=wl.soft_cap)
+    got = mid.float().cpu()
+    assert not torch.isnan(got).any(), "a partial slot was not written"
+    assert torch.equal(torch.isneginf(got[..., D]), torch.isneginf(model[..., D]))
+    fin = ~torch.isneginf(model[..., D])
+    loose = mid_dtype != torch.float32
+    assert_out_close(got[..., :D][fin], model[..., :D][fin], atol=2e-2 if loose else 5e-3, rel=False)
+    assert_lse_close(got[..., D][fin], model[..., D][fin], rtol=1e-2 if loose else 1e-3)
+    assert torch.all(got[..., :D][~fin] == 0)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out, ref)
+    # a 16-bit caller buffer holds the partial LSEs in 16 bits too (the reference's layout, flash_decode.py:239)
+    assert_lse_close(lse, ref_lse, rtol=1e-2 if loose else 1e-3)
+    # internal partials with exactly S splits (16-bit, separate LSE buffer) and the library's own plan agree
+    out_x, lse_x = run_decode(fd, wl, plan_splits=False)
+    assert_out_close(out_x, ref)
+    assert_lse_close(lse_x, ref_lse)
+    if S >= 24:
+        assert 0 < planned < S
+
+
 def test_intra_rank_packs_lse_column(fd):
     wl = _grid_workload(fd, [1320, 18, 463], (32, 8), 128, 16, torch.bfloat16, 0, seed=53)
     g = wl.to(DEV)
