@@ -297,6 +297,18 @@ def test_config5_full_size_every_sequence(fd):
     out64, lse64 = run_decode(fd, wl, plan_splits=False)
     assert_out_rel(out64, out.float(), rms_rtol=5e-3, max_rtol=1e-2)
     assert_lse_close(lse64, lse, rtol=1e-5)
+    # the reference's own partial buffers, [B, Hq, 64, D + 1] in the query's dtype (flash_decode.py:763-766) and in
+    # fp32: rows that start on odd element offsets, large enough (34 / 68 MB) to be written through
+    B, Hq, D = wl.q.shape
+    for mdt in (wl.q.dtype, torch.float32):
+        mid = torch.full((B, Hq, 64, D + 1), float("nan"), dtype=mdt, device=DEV)
+        outv, lsev = run_decode(fd, wl, output_split=mid)
+        assert not torch.isnan(mid).any(), "a partial slot was not written"
+        # a bf16 row holds its LSE in bf16 as well (8 bits of mantissa on a value near 10): the weights of the merge
+        # carry that rounding, which the layout fixes, not the kernel
+        loose = mdt != torch.float32
+        assert_out_rel(outv, out.float(), rms_rtol=2e-2 if loose else 5e-3, max_rtol=5e-2 if loose else 1e-2)
+        assert_lse_close(lsev, lse, rtol=1e-2 if loose else 1e-5)
 
 
 # ---- edge cases
@@ -546,6 +558,30 @@ def test_exact_splits_on_chunked_work_items(fd, kind, S, mid_dtype, soft_cap):
     assert_lse_close(lse_x, ref_lse)
     if S >= 24:
         assert 0 < planned < S
+
+
+@pytest.mark.parametrize("mid_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_partial_buffer_one_element_off_alignment(fd, mid_dtype, D):
+    """A caller's [B, Hq, S, D + 1] partial buffer that starts one element past an aligned address holds the same bits
+    as an aligned one, and the elements on either side of it stay untouched."""
+    lens = [700, 0, 45, 2100]
+    S = 12
+    wl = fd.utils.make_paged_workload("offset_mid", lens, 16, 4, D, 16, torch.bfloat16, S, seed=67)
+    B, Hq = len(lens), 16
+    n = B * Hq * S * (D + 1)
+    flat = torch.full((n + 2,), 7.0, dtype=mid_dtype, device=DEV)
+    mid_off = flat[1:n + 1].view(B, Hq, S, D + 1)
+    mid = torch.full((B, Hq, S, D + 1), float("nan"), dtype=mid_dtype, device=DEV)
+    out_a, lse_a = run_decode(fd, wl, output_split=mid)
+    out_b, lse_b = run_decode(fd, wl, output_split=mid_off)
+    assert flat[0].item() == 7.0 and flat[n + 1].item() == 7.0
+    assert torch.equal(mid.view(torch.uint8 if mid_dtype != torch.float32 else torch.int32),
+                       mid_off.contiguous().view(torch.uint8 if mid_dtype != torch.float32 else torch.int32))
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    ref, ref_lse = oracle_decode(wl)
+    assert_out_close(out_a, ref)
+    assert_lse_close(lse_a, ref_lse, rtol=1e-3 if mid_dtype == torch.float32 else 1e-2)
 
 
 def test_intra_rank_packs_lse_column(fd):

@@ -290,7 +290,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   {
     static const int forced = env_int("FD_STORE_THROUGH");   // tuning override for experiments: 1 always, 2 never
     const int64_t partial_bytes = (int64_t)batch * p->q_heads * p->num_splits * Dv * msz;
-    a.store_through = a.vec_out && forced != 2 && (forced == 1 || partial_bytes >= kStoreThroughBytes) ? 1 : 0;
+    a.store_through = forced != 2 && (forced == 1 || partial_bytes >= kStoreThroughBytes) ? 1 : 0;
   }
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;

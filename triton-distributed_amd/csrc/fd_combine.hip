@@ -174,7 +174,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
 // latency.  Thread (r, c): partials r, r + ROWS, ... and 128-bit column chunk c.  Lane i of every wave loads LSE i
 // (MAXP <= 64 = one per lane); the maximum is a butterfly over the wave and a thread takes the LSEs of its own
 // partials from the lanes that hold them, so nothing goes through LDS before the final sum.
-template <int D, int MAXP, int MID>
+template <int D, int MAXP, int MID, bool VEC>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const CombineArgs a) {
   constexpr int CG = D / 4;
   constexpr int ROWS = kCombineThreads / CG;
@@ -188,17 +188,22 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
   const int h = blockIdx.x - b * a.Hq;
   const int S = a.num_partials;
   const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
-  const float* lse_row = a.mid_lse + ((int64_t)b * a.Hq + h) * S;
   const int r = tid / CG;
   const int c = tid - r * CG;
+  // VEC: rows start on multiples of four elements and a thread owns columns 4c .. 4c + 3 (one 128- or 64-bit load);
+  // else (the reference's [.., D + 1] rows) it owns columns c, c + CG, c + 2 CG, c + 3 CG, so that consecutive
+  // threads still read consecutive elements.
   f32x4 o[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int s = r + p * ROWS;
     o[p] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (s < S) {
-      const int64_t off = mid_base + (int64_t)s * a.s_ms + 4 * c;
-      if constexpr (MID == FD_F32) {
+      const int64_t off = mid_base + (int64_t)s * a.s_ms + (VEC ? 4 * c : c);
+      if constexpr (!VEC) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[p][k] = load_as_f32(a.mid_o, off + k * CG, MID);
+      } else if constexpr (MID == FD_F32) {
         o[p] = *(const f32x4*)((const float*)a.mid_o + off);
       } else {
         const u32x2 w = *(const u32x2*)((const uint16_t*)a.mid_o + off);
@@ -212,7 +217,10 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
       }
     }
   }
-  const float mine = lane < S ? lse_row[lane] : -INFINITY;   // LSE of partial `lane`
+  float mine = -INFINITY;   // LSE of partial `lane`: from its own buffer, or from column D of the partial's row
+  if (lane < S)
+    mine = a.mid_lse ? a.mid_lse[((int64_t)b * a.Hq + h) * S + lane]
+                     : load_as_f32(a.mid_o, mid_base + (int64_t)lane * a.s_ms + D, MID);
   float M = mine;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
@@ -226,7 +234,12 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
     acc += o[p] * wgt;
     L += wgt;
   }
-  *(f32x4*)&s_acc[r][4 * c] = acc;
+  if constexpr (VEC) {
+    *(f32x4*)&s_acc[r][4 * c] = acc;
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) s_acc[r][c + k * CG] = acc[k];
+  }
   if (c == 0) s_l[r] = L;
   __syncthreads();
   if (tid < D) {
@@ -297,7 +310,7 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   // 32 only where there is a workgroup per CU: with few output rows (one long sequence: 96 rows x 42 partials) the
   // general kernel, which spreads a row over several workgroups, is the faster one (5.0 against 5.7 us)
   const int np_own = a.num_partials <= 16 ? 16 : (a.num_partials <= 32 ? 32 : 64);
-  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 && a.vec_mid && a.mid_lse &&
+  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 &&
                      (a.num_partials <= 32 || (a.num_partials <= 64 && rows >= 256));
   // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
   // one workgroup per CU and a thread would still have more than two partials to walk.
@@ -309,7 +322,8 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   const int64_t wgs = small ? rows : rows * (a.D / 4 / cg);
   if (wgs >= ((int64_t)1 << 31)) return FD_ERR_TOO_LARGE;
   const unsigned grid = (unsigned)wgs;
-#define FD_OWN_P(D_, M_) (np_own == 16 ? fd_combine_own_kernel<D_, 16, M_> : np_own == 32 ? fd_combine_own_kernel<D_, 32, M_> : fd_combine_own_kernel<D_, 64, M_>)
+#define FD_OWN_V(D_, M_, V_) (np_own == 16 ? fd_combine_own_kernel<D_, 16, M_, V_> : np_own == 32 ? fd_combine_own_kernel<D_, 32, M_, V_> : fd_combine_own_kernel<D_, 64, M_, V_>)
+#define FD_OWN_P(D_, M_) (a.vec_mid ? FD_OWN_V(D_, M_, true) : FD_OWN_V(D_, M_, false))
 #define FD_OWN(D_) (a.mid_dtype == FD_F32 ? FD_OWN_P(D_, FD_F32) : a.mid_dtype == FD_F16 ? FD_OWN_P(D_, FD_F16) : FD_OWN_P(D_, FD_BF16))
   switch (a.D) {
     case 64: kern = small ? FD_OWN(64) : fd_combine_kernel<64>; break;
@@ -318,6 +332,7 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
     default: return FD_ERR_UNSUPPORTED;
   }
 #undef FD_OWN_P
+#undef FD_OWN_V
 #undef FD_OWN
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;

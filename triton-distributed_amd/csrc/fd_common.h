@@ -217,6 +217,30 @@ __device__ __forceinline__ void store_partial4(void* base, int64_t off, int dtyp
   }
 }
 
+// One value, or two adjacent 16-bit values as one dword (off even, base 4-byte aligned), with the same write-through
+// option and the same restriction as store_partial4.
+__device__ __forceinline__ void store_partial1(void* base, int64_t off, int dtype, float x, bool through) {
+  if (!through) { store_from_f32(base, off, dtype, x); return; }
+  if (dtype == FD_F32) {
+    asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"((float*)base + off), "v"(x) : "memory");
+  } else {
+    const uint32_t w = dtype == FD_F16 ? (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x)
+                                       : (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
+    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"((uint16_t*)base + off), "v"(w) : "memory");
+  }
+}
+__device__ __forceinline__ void store_partial2x16(void* base, int64_t off, int dtype, float x0, float x1, bool through) {
+  const f32x2 v = {x0, x1};
+  const uint32_t w = dtype == FD_F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2))
+                                     : __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  uint16_t* p = (uint16_t*)base + off;
+  if (through) {
+    asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+  } else {
+    *(uint32_t*)p = w;
+  }
+}
+
 // Orders LDS accesses of one wave: lanes of a wave exchange data through LDS
 // without a workgroup barrier (the LDS queue of a wave is in order); this only
 // stops the compiler from moving accesses across the point.
@@ -436,6 +460,45 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
   const int tid = threadIdx.x;
   const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
   constexpr int D4 = D / 4;
+  if (!a.vec_out && !a.tickets) {
+    // Rows that do not start on a multiple of four elements -- the reference's [B, Hq, S, D + 1] layout, whose rows
+    // are D + 1 elements apart: one element per thread, consecutive threads on consecutive elements, so that a store
+    // instruction still covers contiguous memory (256 bytes of fp32 per wave).
+    const int heads = a.member_hb ? HB : nheads;
+    for (int e = tid; e < a.hpw * heads * D; e += nthreads) {
+      const int hm = e / (heads * D);
+      const int r = e - hm * heads * D;
+      const int h = r / D;
+      const int d = r - h * D;
+      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+      const int hb = a.member_hb ? w.hb0 + hm : w.hb;
+      if (h >= a.G - hb * HB) continue;
+      float M = -INFINITY;
+      for (int p = 0; p < w.nsub; ++p) M = fmaxf(M, part[(hm + a.hpw * p) * stride + HB * D + h]);
+      float L = 0.f, o = 0.f;
+      if (M > -INFINITY) {
+        for (int p = 0; p < w.nsub; ++p) {
+          const float* pp = part + (hm + a.hpw * p) * stride;
+          const float wgt = fd_exp2(pp[HB * D + h] - M);
+          L += pp[HB * D + HB + h] * wgt;
+          o += pp[h * D + d] * wgt;
+        }
+      }
+      const float inv = L > 0.f ? 1.0f / L : 0.f;
+      const int head = kvh * a.G + hb * HB + h;
+      const int64_t row = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s;
+      store_partial1(a.out, row + d, a.mid_dtype, o * inv, a.store_through != 0);
+      if (d == 0 && !a.no_lse) {
+        const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+        if (a.lse) {
+          a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
+        } else {
+          store_partial1(a.out, row + D, a.mid_dtype, lse, a.store_through != 0);
+        }
+      }
+    }
+    return;
+  }
   // head blocks as members: the last block of a group may hold fewer heads than the others
   const int per_head = (a.member_hb ? HB : nheads) * D4;
   for (int e = tid; e < a.hpw * per_head; e += nthreads) {
@@ -498,6 +561,55 @@ __device__ __forceinline__ void wave_store_partial(const SplitArgs& a, const flo
   constexpr int D4 = D / 4;          // lanes per row
   constexpr int RPI = 64 / D4;       // rows per store instruction
   static_assert(D4 <= 64 && HB % RPI == 0, "one wave covers whole rows");
+  if (!a.vec_out) {
+    // rows that do not start on a multiple of four elements (the reference's D + 1 layout): one element per lane,
+    // 64 consecutive elements per store instruction
+    for (int h = 0; h < nheads; ++h) {
+      float inv = 0.f, lse = -INFINITY;
+      if (!empty) {
+        const float M = part[HB * D + h];
+        const float L = part[HB * D + HB + h];
+        inv = L > 0.f ? 1.0f / L : 0.f;
+        lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+      }
+      const int head = head0 + h;
+      const int64_t row = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s;
+      const bool through = a.store_through != 0;
+      if (a.mid_dtype != FD_F32 && !a.lse && !a.no_lse) {
+        // 16-bit row of D values and the LSE behind them: dword stores of two values on 4-byte boundaries.  A row
+        // that starts between two boundaries stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that
+        // starts on a boundary pairs (0, 1) .. (D - 2, D - 1) and stores the LSE alone.
+        const int first = (int)(((reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row) & 1);
+#pragma unroll
+        for (int k = 0; k < (D / 2 + 63) / 64; ++k) {
+          const int pr = lane + 64 * k;
+          if (pr < D / 2) {
+            const int e = 2 * pr + first;
+            const float x0 = empty ? 0.f : part[h * D + e] * inv;
+            const float x1 = e + 1 == D ? lse : (empty ? 0.f : part[h * D + e + 1] * inv);
+            store_partial2x16(a.out, row + e, a.mid_dtype, x0, x1, through);
+          }
+        }
+        if (lane == 0)
+          store_partial1(a.out, row + (first ? 0 : D), a.mid_dtype,
+                         first ? (empty ? 0.f : part[h * D] * inv) : lse, through);
+        continue;
+      }
+#pragma unroll
+      for (int k = 0; k < D / 64; ++k) {
+        const int d = lane + 64 * k;
+        store_partial1(a.out, row + d, a.mid_dtype, empty ? 0.f : part[h * D + d] * inv, through);
+      }
+      if (lane == 0 && !a.no_lse) {
+        if (a.lse) {
+          a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
+        } else {
+          store_partial1(a.out, row + D, a.mid_dtype, lse, through);
+        }
+      }
+    }
+    return;
+  }
   const int d = (lane % D4) * 4;
 #pragma unroll
   for (int r = 0; r < HB / RPI; ++r) {
