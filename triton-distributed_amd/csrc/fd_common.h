@@ -549,6 +549,11 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
   }
 }
 
+// Values one lane holds of a D-wide row in wave_store_partial's element-wise forms: 64 lanes x 1 value (or x 2 values
+// for the 16-bit pairs) per pass.
+template <int D>
+__host__ __device__ constexpr int paired_values_per_lane() { return D <= 128 ? 2 : D / 64; }
+
 // Chunked work items: ONE wave stores the finished partial of split s for its own HB head slots, from an LDS buffer
 // `part` of its own (same layout as one wave's slice in cta_merge_store; the wave has ordered its LDS writes before
 // the call).  Called at the end of the wave's run only: on this target stores and loads of a wave retire in order
@@ -562,49 +567,75 @@ __device__ __forceinline__ void wave_store_partial(const SplitArgs& a, const flo
   constexpr int RPI = 64 / D4;       // rows per store instruction
   static_assert(D4 <= 64 && HB % RPI == 0, "one wave covers whole rows");
   if (!a.vec_out) {
-    // rows that do not start on a multiple of four elements (the reference's D + 1 layout): one element per lane,
-    // 64 consecutive elements per store instruction
-    for (int h = 0; h < nheads; ++h) {
-      float inv = 0.f, lse = -INFINITY;
-      if (!empty) {
-        const float M = part[HB * D + h];
-        const float L = part[HB * D + HB + h];
-        inv = L > 0.f ? 1.0f / L : 0.f;
-        lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
-      }
-      const int head = head0 + h;
-      const int64_t row = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s;
-      const bool through = a.store_through != 0;
-      if (a.mid_dtype != FD_F32 && !a.lse && !a.no_lse) {
-        // 16-bit row of D values and the LSE behind them: dword stores of two values on 4-byte boundaries.  A row
-        // that starts between two boundaries stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that
-        // starts on a boundary pairs (0, 1) .. (D - 2, D - 1) and stores the LSE alone.
-        const int first = (int)(((reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row) & 1);
-#pragma unroll
-        for (int k = 0; k < (D / 2 + 63) / 64; ++k) {
-          const int pr = lane + 64 * k;
-          if (pr < D / 2) {
-            const int e = 2 * pr + first;
-            const float x0 = empty ? 0.f : part[h * D + e] * inv;
-            const float x1 = e + 1 == D ? lse : (empty ? 0.f : part[h * D + e + 1] * inv);
-            store_partial2x16(a.out, row + e, a.mid_dtype, x0, x1, through);
-          }
-        }
-        if (lane == 0)
-          store_partial1(a.out, row + (first ? 0 : D), a.mid_dtype,
-                         first ? (empty ? 0.f : part[h * D] * inv) : lse, through);
-        continue;
-      }
-#pragma unroll
-      for (int k = 0; k < D / 64; ++k) {
-        const int d = lane + 64 * k;
-        store_partial1(a.out, row + d, a.mid_dtype, empty ? 0.f : part[h * D + d] * inv, through);
-      }
-      if (lane == 0 && !a.no_lse) {
+    // Rows that do not start on a multiple of four elements (the reference's D + 1 layout): consecutive lanes on
+    // consecutive elements, so that a store instruction covers contiguous memory.  A 16-bit row of D values with the
+    // LSE behind them goes out as dwords of two values on 4-byte boundaries: a row that starts between two boundaries
+    // stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that starts on a boundary pairs (0, 1) ..
+    // (D - 2, D - 1) and stores the LSE alone.
+    const bool through = a.store_through != 0;
+    const bool paired = a.mid_dtype != FD_F32 && !a.lse && !a.no_lse;
+    const int64_t row0 = (int64_t)b * a.so_b + (int64_t)head0 * a.so_h + (int64_t)s * a.so_s;
+    const uint64_t par0 = (reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row0;
+    // lane h holds row h's scale and LSE (one LDS round trip for all rows) and stores the row's single value
+    const int hl = lane < nheads ? lane : nheads - 1;
+    float inv_l = 0.f, lse_l = -INFINITY, x0_l = 0.f;
+    if (!empty) {
+      const float M = part[HB * D + hl];
+      const float L = part[HB * D + HB + hl];
+      inv_l = L > 0.f ? 1.0f / L : 0.f;
+      lse_l = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+      x0_l = part[hl * D] * inv_l;
+    }
+    if (lane < nheads) {
+      const int64_t row_l = row0 + (int64_t)hl * a.so_h;
+      if (paired) {
+        const bool first_l = ((par0 + (uint64_t)hl * (uint64_t)a.so_h) & 1) != 0;
+        store_partial1(a.out, row_l + (first_l ? 0 : D), a.mid_dtype, first_l ? x0_l : lse_l, through);
+      } else if (!a.no_lse) {
         if (a.lse) {
-          a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
+          a.lse[((int64_t)b * a.Hq + head0 + hl) * a.S + s] = lse_l;
         } else {
-          store_partial1(a.out, row + D, a.mid_dtype, lse, through);
+          store_partial1(a.out, row_l + D, a.mid_dtype, lse_l, through);
+        }
+      }
+    }
+    // four rows at a time: their values are requested from LDS together
+    constexpr int NV = paired_values_per_lane<D>();
+    for (int h0 = 0; h0 < nheads; h0 += 4) {
+      float x[4][NV];
+      float inv[4], lse[4];
+      int first[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int hh = min(h0 + i, nheads - 1);
+        inv[i] = __shfl(inv_l, hh);
+        lse[i] = __shfl(lse_l, hh);
+        first[i] = paired ? (int)((par0 + (uint64_t)hh * (uint64_t)a.so_h) & 1) : 0;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+          // paired: values 2 (lane + 64 (k / 2)) + first + (k & 1); else lane + 64 k
+          const int e = paired ? 2 * (lane + 64 * (k >> 1)) + first[i] + (k & 1) : lane + 64 * k;
+          x[i][k] = empty || e >= D ? 0.f : part[hh * D + e];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (h0 + i >= nheads) break;
+        const int64_t row = row0 + (int64_t)(h0 + i) * a.so_h;
+        if (paired) {
+#pragma unroll
+          for (int k = 0; k < NV; k += 2) {
+            const int e = 2 * (lane + 64 * (k >> 1)) + first[i];
+            if (e < D)
+              store_partial2x16(a.out, row + e, a.mid_dtype, x[i][k] * inv[i],
+                                e + 1 == D ? lse[i] : x[i][k + 1] * inv[i], through);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < NV; ++k) {
+            const int e = lane + 64 * k;
+            if (e < D) store_partial1(a.out, row + e, a.mid_dtype, x[i][k] * inv[i], through);
+          }
         }
       }
     }
