@@ -6,6 +6,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 #include <stdint.h>
 
 #include "../../include/flash_decode.h"
@@ -502,25 +504,58 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
   // head blocks as members: the last block of a group may hold fewer heads than the others
   const int per_head = (a.member_hb ? HB : nheads) * D4;
   for (int e = tid; e < a.hpw * per_head; e += nthreads) {
-    const int hm = e / per_head;
-    const int r = e - hm * per_head;
+    int hm = 0, r = e;
+    while (r >= per_head) {   // at most hpw - 1 <= 3 rounds: cheaper than a division by a run-time value
+      r -= per_head;
+      ++hm;
+    }
     const int h = r / D4;
     const int d = (r - h * D4) * 4;
     const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
     const int hb = a.member_hb ? w.hb0 + hm : w.hb;
     if (h >= a.G - hb * HB) continue;
-    float M = -INFINITY;
-    for (int p = 0; p < w.nsub; ++p) M = fmaxf(M, part[(hm + a.hpw * p) * stride + HB * D + h]);
-    float L = 0.f;
+    // This runs once per workgroup, after the last tile, with nothing left to overlap: every LDS read below is
+    // requested before the first one is used (unrolled over the sub-ranges; a loop over a run-time count takes one
+    // dependent LDS round trip per sub-range and value, about 1 us per launch in all).
+    float M = -INFINITY, L = 0.f;
     f32x4 o = {0.f, 0.f, 0.f, 0.f};
-    if (M > -INFINITY) {
-      for (int p = 0; p < w.nsub; ++p) {
+    auto merge = [&](auto nsub_tag) {
+      constexpr int NS = decltype(nsub_tag)::value;
+      float mm[NS], ll[NS];
+      f32x4 xx[NS];
+#pragma unroll
+      for (int p = 0; p < NS; ++p) {
         const float* pp = part + (hm + a.hpw * p) * stride;
-        float wgt = fd_exp2(pp[HB * D + h] - M);  // exp2(-inf) = 0 for idle waves
-        L += pp[HB * D + HB + h] * wgt;
-        f32x4 x = *(const f32x4*)(pp + h * D + d);
-        o += x * wgt;
+        mm[p] = pp[HB * D + h];
+        ll[p] = pp[HB * D + HB + h];
+        xx[p] = *(const f32x4*)(pp + h * D + d);
       }
+#pragma unroll
+      for (int p = 0; p < NS; ++p) M = fmaxf(M, mm[p]);
+      if (M > -INFINITY) {
+#pragma unroll
+        for (int p = 0; p < NS; ++p) {
+          const float wgt = fd_exp2(mm[p] - M);  // exp2(-inf) = 0 for idle waves
+          L += ll[p] * wgt;
+          o += xx[p] * wgt;
+        }
+      }
+    };
+    switch (w.nsub) {
+      case 1: merge(std::integral_constant<int, 1>{}); break;
+      case 2: merge(std::integral_constant<int, 2>{}); break;
+      case 4: merge(std::integral_constant<int, 4>{}); break;
+      case 8: merge(std::integral_constant<int, 8>{}); break;
+      default:
+        for (int p = 0; p < w.nsub; ++p) M = fmaxf(M, part[(hm + a.hpw * p) * stride + HB * D + h]);
+        if (M > -INFINITY) {
+          for (int p = 0; p < w.nsub; ++p) {
+            const float* pp = part + (hm + a.hpw * p) * stride;
+            const float wgt = fd_exp2(pp[HB * D + h] - M);
+            L += pp[HB * D + HB + h] * wgt;
+            o += *(const f32x4*)(pp + h * D + d) * wgt;
+          }
+        }
     }
     float inv = L > 0.f ? 1.0f / L : 0.f;
     o *= inv;
