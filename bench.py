@@ -389,8 +389,8 @@ def main():
     p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_bound, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
                         wl.k_scale, wl.v_scale, args.path, args.waves)
     p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials
-    p.mid_dtype = fk.internal_partial_dtype(out.dtype, not args.exact_splits, args.fuse)
     S_eff = S_bound if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
+    p.mid_dtype = fk.internal_partial_dtype(out.dtype, not args.exact_splits, args.fuse, B * Hq * S_eff * D)
     if not args.exact_splits:
         p.split_adapt = lib.fd_plan_min_splits(byref(p), B)
     p.num_splits = S_eff

@@ -38,6 +38,8 @@ which is the same thing for the fp16 inputs its tests use).
 """
 from __future__ import annotations
 
+import os
+
 from ctypes import byref
 from typing import Optional
 
@@ -86,13 +88,19 @@ def auto_split_bound(capacity: int) -> int:
     return max(DEFAULT_KV_SPLITS, min(MAX_AUTO_KV_SPLITS, capacity // 512))
 
 
-def internal_partial_dtype(out_dtype, plan_splits, fuse_combine):
+PARTIALS_16BIT_FROM_BYTES = int(os.environ.get("FD_PARTIALS_16BIT_FROM_BYTES", 4 << 20))
+
+
+def internal_partial_dtype(out_dtype, plan_splits, fuse_combine, partial_elems=0):
     """Element type of the partials when they stay inside the library (the LSEs are always fp32, in their own
-    buffer).  Planned splits are few and long: fp32.  A caller who insists on exactly ``kv_split`` splits
-    (``plan_splits=False``) gets partials in the output's precision when that is 16-bit -- what the reference's
-    intra-rank wrapper allocates (flash_decode.py:867-868; the plain one fp16 whatever the inputs, :783-784): with 32
-    or 64 splits per sequence the partials are megabytes that the split kernel writes and the combine reads back."""
-    if plan_splits or fuse_combine or out_dtype not in (torch.float16, torch.bfloat16):
+    buffer).  Planned splits are few and long: fp32, unless there are ``PARTIALS_16BIT_FROM_BYTES`` of them or more
+    (many query heads per KV head, large batches).  Those, and the partials of a caller who insists on exactly
+    ``kv_split`` splits (``plan_splits=False``), take the output's precision when that is 16-bit -- what the
+    reference's intra-rank wrapper allocates (flash_decode.py:867-868; the plain one fp16 whatever the inputs,
+    :783-784): megabytes that the split kernel writes at its very end and the combine reads back."""
+    if fuse_combine or out_dtype not in (torch.float16, torch.bfloat16):
+        return FD_F32
+    if plan_splits and 4 * partial_elems < PARTIALS_16BIT_FROM_BYTES:
         return FD_F32
     return FD_F16 if out_dtype == torch.float16 else FD_BF16
 
@@ -259,7 +267,7 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         mid_ptr = hold.data_ptr() if hold is not None else None
         lse_split_ptr = mid_ptr + 4 * n_o if hold is not None else None
         mid_dtype = internal_partial_dtype(output_combine.dtype if output_combine is not None else q.dtype,
-                                           plan_splits, fuse_combine)
+                                           plan_splits, fuse_combine, n_o)
         so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
     else:
         assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
