@@ -456,8 +456,160 @@ __device__ __forceinline__ int token_row(const SplitArgs& a, const int32_t* bt_r
 // heads, a head block of the one KV head.  Called by every thread of the workgroup after a __syncthreads() with
 // nheads = the calling wave's head count.  fp8 caches: the waves have already multiplied their accumulators by
 // v_scale[kv head] (a load here, between the stores, would cost its latency once per loop iteration).
+//
+// Two steps with a barrier between them.  First one thread per (member, head) row turns the row's running maxima
+// into merge weights 2^(m_p - M) in place, leaves 1 / L in sub-range 0's sum slot and stores the row's LSE; then every
+// thread sums its four (or, for rows that do not start on a multiple of four elements, its one) output values over
+// the sub-ranges with those weights.  All of this runs once per workgroup after the last tile, with nothing left to
+// overlap it: the per-row arithmetic is not repeated per value (a workgroup of 2 x 32 heads merged for 4.6 us when
+// every thread derived its row's weights itself, 8 rounds of about 200 instructions), and every LDS read of a
+// round is requested before the first one is used (unrolled over the sub-ranges).
 template <int HB, int D>
-__device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float* part, int stride,
+__device__ __forceinline__ void cta_merge_store_rounds(const SplitArgs& a, float* part, int stride, const WorkItem& w,
+                                                int nheads) {
+  const int tid = threadIdx.x;
+  const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
+  constexpr int D4 = D / 4;
+  // head blocks as members: the last block of a group may hold fewer heads than the others
+  const int heads = a.member_hb ? HB : nheads;
+  const int pstep = a.hpw * stride;   // floats between the partials of two sub-ranges of one member
+  const bool through = a.store_through != 0;
+
+  // ---- step 1: weights, 1 / L and the LSE of every row
+  for (int row = tid; row < a.hpw * heads; row += nthreads) {
+    int hm = 0;   // member of the row, without a division by a run-time value or a divergent loop (hpw <= 8)
+#pragma unroll
+    for (int k = 1; k < 8; ++k) hm += row >= k * heads;
+    const int h = row - hm * heads;
+    float* ml = part + hm * stride + HB * D + h;   // m_p at ml[p * pstep], l_p at ml[p * pstep + HB]
+    float M = -INFINITY, L = 0.f;
+    auto weigh = [&](auto nsub_tag, int ns) {
+      constexpr int NS = decltype(nsub_tag)::value;   // 0: run-time count ns
+      constexpr int CAP = NS ? NS : 1;
+      float mm[CAP], ll[CAP];
+      if constexpr (NS > 0) {
+#pragma unroll
+        for (int p = 0; p < NS; ++p) {
+          mm[p] = ml[p * pstep];
+          ll[p] = ml[p * pstep + HB];
+        }
+#pragma unroll
+        for (int p = 0; p < NS; ++p) M = fmaxf(M, mm[p]);
+#pragma unroll
+        for (int p = 0; p < NS; ++p) {
+          const float wgt = M > -INFINITY ? fd_exp2(mm[p] - M) : 0.f;   // exp2(-inf) = 0 for idle waves
+          L += ll[p] * wgt;
+          ml[p * pstep] = wgt;
+        }
+      } else {
+        for (int p = 0; p < ns; ++p) M = fmaxf(M, ml[p * pstep]);
+        for (int p = 0; p < ns; ++p) {
+          const float wgt = M > -INFINITY ? fd_exp2(ml[p * pstep] - M) : 0.f;
+          L += ml[p * pstep + HB] * wgt;
+          ml[p * pstep] = wgt;
+        }
+      }
+    };
+    switch (w.nsub) {
+      case 1: weigh(std::integral_constant<int, 1>{}, 1); break;
+      case 2: weigh(std::integral_constant<int, 2>{}, 2); break;
+      case 4: weigh(std::integral_constant<int, 4>{}, 4); break;
+      case 8: weigh(std::integral_constant<int, 8>{}, 8); break;
+      default: weigh(std::integral_constant<int, 0>{}, w.nsub);
+    }
+    ml[HB] = L > 0.f ? 1.0f / L : 0.f;
+    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+    const int hb = a.member_hb ? w.hb0 + hm : w.hb;
+    if (h < a.G - hb * HB && (a.tickets || !a.no_lse)) {
+      const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+      const int head = kvh * a.G + hb * HB + h;
+      const int64_t lse_at = ((int64_t)w.b * a.Hq + head) * a.S + w.s;
+      const int64_t col_d = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + D;
+      if (a.tickets) {   // fused combine (fp32 partials only): another XCD's workgroup may read these
+        store_f32_agent(a.lse ? a.lse + lse_at : (float*)a.out + col_d, lse);
+      } else if (a.lse) {
+        a.lse[lse_at] = lse;
+      } else {
+        store_partial1(a.out, col_d, a.mid_dtype, lse, through);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- step 2: the values.  V values per thread and round: 4 (one 128- or 64-bit store), or 1 where rows do not
+  // start on a multiple of four elements (the reference's [B, Hq, S, D + 1] layout): consecutive threads on
+  // consecutive elements, so that a store instruction still covers contiguous memory.
+  // The loop is specialised on everything that is the same for all its rounds (values per thread, sub-range count):
+  // a taken branch costs a wave an instruction-buffer refill, and with the decisions inside the loop a round was
+  // some 25 of them -- about 1100 cycles per round for 80 instructions of work.
+  auto values = [&](auto vec_tag, auto nsub_tag, int ns) {
+    constexpr int V = decltype(vec_tag)::value;
+    constexpr int NS = decltype(nsub_tag)::value;   // 0: run-time count ns
+    constexpr int PER_ROW = D / V;
+    using Val = typename std::conditional<V == 4, f32x4, float>::type;
+    const int per_member = heads * PER_ROW;
+    const bool fused = a.tickets != nullptr;
+    for (int e = tid; e < a.hpw * per_member; e += nthreads) {
+      // member of e without a division by a run-time value or a divergent loop (hpw <= 8)
+      int hm = 0;
+#pragma unroll
+      for (int k = 1; k < 8; ++k) hm += e >= k * per_member;
+      const int r = e - hm * per_member;
+      const int h = r / PER_ROW;
+      const int d = (r - h * PER_ROW) * V;
+      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+      const int hb = a.member_hb ? w.hb0 + hm : w.hb;
+      if (h >= a.G - hb * HB) continue;
+      const float* x0 = part + hm * stride + h * D + d;
+      const float* w0 = part + hm * stride + HB * D + h;
+      Val o{};
+      const float inv = w0[HB];   // 1 / L
+      if constexpr (NS > 0) {
+        Val xx[NS];
+        float ww[NS];
+#pragma unroll
+        for (int p = 0; p < NS; ++p) {
+          xx[p] = *(const Val*)(x0 + p * pstep);
+          ww[p] = w0[p * pstep];
+        }
+#pragma unroll
+        for (int p = 0; p < NS; ++p) o += xx[p] * ww[p];
+      } else {
+        for (int p = 0; p < ns; ++p) o += *(const Val*)(x0 + p * pstep) * w0[p * pstep];
+      }
+      o *= inv;
+      const int head = kvh * a.G + hb * HB + h;
+      const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;
+      if constexpr (V == 4) {
+        if (fused) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) store_f32_agent((float*)a.out + off + i, o[i]);
+        } else {
+          store_partial4(a.out, off, a.mid_dtype, o, through);
+        }
+      } else {
+        store_partial1(a.out, off, a.mid_dtype, o, through);
+      }
+    }
+  };
+  auto values_of = [&](auto vec_tag) {
+    switch (w.nsub) {
+      case 1: values(vec_tag, std::integral_constant<int, 1>{}, 1); break;
+      case 2: values(vec_tag, std::integral_constant<int, 2>{}, 2); break;
+      case 4: values(vec_tag, std::integral_constant<int, 4>{}, 4); break;
+      case 8: values(vec_tag, std::integral_constant<int, 8>{}, 8); break;
+      default: values(vec_tag, std::integral_constant<int, 0>{}, w.nsub);
+    }
+  };
+  if (a.vec_out || a.tickets) {
+    values_of(std::integral_constant<int, 4>{});
+  } else {
+    values_of(std::integral_constant<int, 1>{});
+  }
+}
+
+template <int HB, int D>
+__device__ __forceinline__ void cta_merge_store_one_round(const SplitArgs& a, const float* part, int stride,
                                                 const WorkItem& w, int nheads) {
   const int tid = threadIdx.x;
   const int nthreads = 64 * a.hpw * a.nsub;   // == blockDim.x, without a trip to the implicit kernel arguments
@@ -581,6 +733,19 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, const float*
         }
       }
     }
+  }
+}
+
+// Few rows (at most two rounds of four values per thread): every thread derives its row's weights itself, no second
+// barrier (config 2, 2 x 4 heads: 44.5 us per step against 44.9 us with the two steps below).  More rows: two steps.
+template <int HB, int D>
+__device__ __forceinline__ void cta_merge_store(const SplitArgs& a, float* part, int stride, const WorkItem& w,
+                                                int nheads) {
+  const int heads = a.member_hb ? HB : nheads;
+  if (a.hpw * heads * (D / 4) <= 2 * 64 * a.hpw * a.nsub) {
+    cta_merge_store_one_round<HB, D>(a, part, stride, w, nheads);
+  } else {
+    cta_merge_store_rounds<HB, D>(a, part, stride, w, nheads);
   }
 }
 

@@ -343,7 +343,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
     // ---- wave result -> LDS, then workgroup merge
     stage_partial(part);
     __syncthreads();
-    cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
+    cta_merge_store<kHB, kD>(a, (float*)smem, kWaveLds / 4, w, nheads);
     if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
   }
 }

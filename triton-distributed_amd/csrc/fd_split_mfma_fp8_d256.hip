@@ -223,7 +223,7 @@ __global__ void __launch_bounds__(512) fd_split_mfma_fp8_d256_kernel(const Split
   }
   __syncthreads();
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
+  cta_merge_store<kHB, kD>(a, (float*)smem, kWaveLds / 4, w, nheads);
   if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);
 }
 

@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(KH == 2 ? 256 : 512) __attribute__((amdgpu_wav
   }
   __syncthreads();
   const int nheads = KH == 2 ? a.G : min(16, a.G - w.hb * 16);
-  cta_merge_store<kHB, kD>(a, (const float*)smem, kWaveLds / 4, w, nheads);
+  cta_merge_store<kHB, kD>(a, (float*)smem, kWaveLds / 4, w, nheads);
   if (a.tickets) fused_combine<kD>(a, w, w.kvh * a.G + w.hb * kHB, nheads, (float*)smem);  // hpw == 1 when fused
 }
 

@@ -297,7 +297,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
     }
   }
   __syncthreads();
-  cta_merge_store<GH, DV>(a, (const float*)smem, PART, w, nheads);
+  cta_merge_store<GH, DV>(a, (float*)smem, PART, w, nheads);
   if (a.tickets) fused_combine<DV>(a, w, head0, nheads, (float*)smem);  // hpw == 1 when fused
 }
 
