@@ -560,6 +560,47 @@ def test_exact_splits_on_chunked_work_items(fd, kind, S, mid_dtype, soft_cap):
         assert 0 < planned < S
 
 
+# ---- the library's own partial layout on the chunked path: rows [B, Hq, S, D] on multiples of four elements and the
+# LSEs in their own fp32 buffer.  A wave then parks finished (normalised, mid-dtype) partials and walks up to four splits;
+# every partial against the per-split model, through the C ABI's split entry point
+@pytest.mark.parametrize("kind", ["bf16", "fp16_g32", "fp8", "bf16_g8"])
+@pytest.mark.parametrize("S,mid_dtype", [(64, torch.bfloat16), (32, torch.float32), (27, torch.float16), (5, torch.bfloat16)])
+def test_exact_splits_internal_layout_every_partial(fd, kind, S, mid_dtype):
+    from ctypes import byref
+    fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
+    Hq, Hkv, dtype, fp8 = {"bf16": (32, 8, torch.bfloat16, False), "fp16_g32": (128, 4, torch.float16, False),
+                           "fp8": (64, 8, torch.bfloat16, True), "bf16_g8": (64, 8, torch.bfloat16, False)}[kind]
+    lens = [8200, 18, 0, 1, 4097, 777, 64, 2500]
+    D = 128
+    wl = fd.utils.make_paged_workload("internal_" + kind, lens, Hq, Hkv, D, 16, dtype, S, seed=71 + S, fp8_kv=fp8)
+    g = wl.to(DEV)
+    B = len(lens)
+    L = fd._lib
+    lib = fd.load_library()
+    p = fk._make_params(g.q, g.k_cache, g.block_table, S, 0.0, L.fd_dtype_of(torch.empty(0, dtype=mid_dtype)),
+                        L.fd_dtype_of(g.q), g.k_scale, g.v_scale, "auto", 0)
+    mid = torch.full((B, Hq, S, D), float("nan"), dtype=mid_dtype, device=DEV)
+    lse = torch.full((B, Hq, S), float("nan"), dtype=torch.float32, device=DEV)
+    L.check(lib.fd_split_kv(
+        torch.cuda.current_stream().cuda_stream, g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(),
+        mid.data_ptr(), lse.data_ptr(), float(g.scale), g.block_table.data_ptr(), g.kv_lens.data_ptr(), B,
+        g.q.stride(0), g.q.stride(1), g.k_cache.stride(-3), g.k_cache.stride(-2), g.v_cache.stride(-3),
+        g.v_cache.stride(-2), mid.stride(0), mid.stride(1), mid.stride(2), g.block_table.stride(0), None, byref(p)))
+    torch.cuda.synchronize()
+    kc, vc = wl.k_cache, wl.v_cache
+    if fp8:
+        kc = oracle.dequant_fp8_cache(kc.view(torch.uint8), wl.k_scale)
+        vc = oracle.dequant_fp8_cache(vc.view(torch.uint8), wl.v_scale)
+    model = oracle.model_split_kv(wl.q.float(), kc.float(), vc.float(), lens, wl.block_table, wl.scale, S)
+    got, got_lse = mid.float().cpu(), lse.cpu()
+    assert not torch.isnan(got).any() and not torch.isnan(got_lse).any(), "a partial slot was not written"
+    assert torch.equal(torch.isneginf(got_lse), torch.isneginf(model[..., D]))
+    fin = ~torch.isneginf(model[..., D])
+    assert_out_close(got[fin], model[..., :D][fin], atol=2e-2 if mid_dtype != torch.float32 else 5e-3, rel=False)
+    assert_lse_close(got_lse[fin], model[..., D][fin], rtol=1e-3)
+    assert torch.all(got[~fin] == 0)
+
+
 @pytest.mark.parametrize("mid_dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("D", [64, 128, 256])
 def test_partial_buffer_one_element_off_alignment(fd, mid_dtype, D):

@@ -106,6 +106,8 @@ constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most
 constexpr int64_t kStoreThroughBytes = 16 << 20;   // partials of a step from which on they are written through
 constexpr int kMaxChunkBatch = 32;     // chunked work items: largest batch they are used for
 constexpr int kMaxSplitsPerWave = 2;   // chunked work items: splits one wave walks (all but the last parked in LDS)
+constexpr int kMaxSplitsPerWaveFinal = 4;   // ... when a parked partial is the finished one (a quarter to an eighth of the bytes)
+constexpr int kChunkLdsBytes = 80 * 1024;   // LDS a chunked workgroup may take: two of them per CU
 
 int env_waves() {
   static const int v = env_int("FD_WAVES_PER_BLOCK");
@@ -116,6 +118,9 @@ int env_heads() {
   return v;
 }
 // FD_NO_CHUNK=1 (experiments): one workgroup per split even where a workgroup could walk several.
+// LDS of one wave's staging buffer in the head_dim-128 MFMA kernels (the larger of the 16-bit and the fp8 kernel's)
+int hb_slots_lds(int hbsz) { return hbsz > 16 ? (32 * 128 + 2 * 32) * 4 : 64 * 144; }
+
 bool env_no_chunk() {
   static const int v = env_int("FD_NO_CHUNK");
   return v != 0;
@@ -357,16 +362,23 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   const int64_t wave_target = use_mfma && !(kv_fp8 && D == 64 && !pair) ? kTargetWaves : kTargetWavesValu;
   int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
                                  : choose_waves(wgs, max_tok_split, tile, wave_target, max_waves);
+  int chunk_per_wave = 1;
   if (a.chunk > 1) {
     // The waves of a head take whole splits, kMaxSplitsPerWave at most: a wave keeps the finished partials of all but
     // its last split in LDS until it has issued its last load (stores and loads of a wave retire in order, so a store
     // between two tiles would hold back the loads behind it).
     while (waves > 1 && waves > a.chunk) waves >>= 1;
-    int per_wave = (a.chunk + waves - 1) / waves;
-    if (per_wave > kMaxSplitsPerWave) per_wave = kMaxSplitsPerWave;
-    a.chunk = waves * per_wave;
-    a.park = per_wave - 1;
-    if (a.chunk == 1) a.park = 0;
+    // Partials with rows on multiples of four elements (the library's own layout) are parked finished -- normalised,
+    // in mid_dtype, the rows of the real heads only: 2 KB for 8 heads in bf16 against 8.3 KB of raw state -- and a
+    // wave walks up to four splits; else the raw state is parked and normalised when it is stored.
+    const int hb_slots = a.hbsz > 16 ? 32 : 16;
+    a.park_final = a.vec_out;
+    a.park_bytes = a.park_final ? hb_slots * 4 + a.hbsz * D * msz : (hb_slots * D + 2 * hb_slots) * 4;
+    chunk_per_wave = (a.chunk + waves - 1) / waves;
+    const int cap = a.park_final ? kMaxSplitsPerWaveFinal : kMaxSplitsPerWave;
+    if (chunk_per_wave > cap) chunk_per_wave = cap;
+    a.chunk = waves * chunk_per_wave;
+    a.park = chunk_per_wave - 1;
   }
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
   a.hpw = 1;
@@ -383,6 +395,15 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     }
   } else if (use_mfma && !fuse) {
     a.hpw = choose_heads_per_group(a.Hkv, D * kvsz * (pair ? 2 : 1), waves, wgs, max_waves);
+  }
+  if (a.chunk > 1) {
+    // two chunked workgroups per CU: fewer parked splits per wave if their LDS would not allow it
+    const int wave_lds = hb_slots_lds(a.hbsz);
+    while (chunk_per_wave > 1 &&
+           (int64_t)a.hpw * waves * (wave_lds + (int64_t)(chunk_per_wave - 1) * a.park_bytes) > kChunkLdsBytes)
+      --chunk_per_wave;
+    a.chunk = waves * chunk_per_wave;
+    a.park = chunk_per_wave - 1;
   }
   a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / a.hpw * a.nhb;
   a.nsub = waves;

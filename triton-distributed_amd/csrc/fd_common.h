@@ -66,6 +66,10 @@ struct SplitArgs {
   int32_t store_through;          // 1: partials are written through to memory (sc0 sc1) instead of being left dirty in
                                   // the XCD's L2 until the kernel ends; pays off for tens of MB of partials
   int32_t park;                   // chunked work items: finished partials a wave parks in LDS besides its last one
+  int32_t park_final;             // 1: a parked partial is the finished one -- fp32 LSEs of the wave's head slots, then
+                                  // normalised rows [head][D] in mid_dtype (rows that start on multiples of four
+                                  // elements only); 0: the wave's raw state in cta_merge_store's layout
+  int32_t park_bytes;             // LDS bytes of one parked partial
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
   int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
@@ -746,6 +750,72 @@ __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, float* part,
     cta_merge_store_one_round<HB, D>(a, part, stride, w, nheads);
   } else {
     cta_merge_store_rounds<HB, D>(a, part, stride, w, nheads);
+  }
+}
+
+// Eight consecutive values of a finished partial row into a parked slot's rows (SplitArgs::park_final): two 128-bit
+// LDS writes for fp32, one of eight packed values for fp16 / bf16.  elem = element offset of the first value.
+__device__ __forceinline__ void park_store8(char* rows, int elem, int dtype, const float (&v)[8]) {
+  if (dtype == FD_F32) {
+    float* p = (float*)rows + elem;
+    *(f32x4*)p = f32x4{v[0], v[1], v[2], v[3]};
+    *(f32x4*)(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+  } else {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const f32x2 x = {v[2 * e], v[2 * e + 1]};
+      w[e] = dtype == FD_F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2))
+                             : __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    }
+    *(u32x4*)((uint16_t*)rows + elem) = w;
+  }
+}
+
+// Chunked work items, SplitArgs::park_final: ONE wave copies a finished partial that it parked in LDS (HB fp32 LSEs,
+// then rows [head][D] in mid_dtype) to split s of its head slots.  Same geometry as wave_store_partial: four values
+// per lane, whole rows per store instruction.
+template <int HB, int D>
+__device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char* slot, int b, int head0, int nheads,
+                                                 int s) {
+  const int lane = threadIdx.x & 63;
+  constexpr int D4 = D / 4;
+  constexpr int RPI = 64 / D4;
+  const float* lse_slot = (const float*)slot;
+  const char* rows = slot + HB * 4;
+  const int d = (lane % D4) * 4;
+  const bool through = a.store_through != 0;
+#pragma unroll
+  for (int r = 0; r < HB / RPI; ++r) {
+    const int h = r * RPI + lane / D4;
+    if (h >= nheads) continue;
+    const int head = head0 + h;
+    const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
+    if (a.mid_dtype == FD_F32) {
+      const f32x4 v = *(const f32x4*)((const float*)rows + h * D + d);
+      float* p = (float*)a.out + off;
+      if (through) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+      } else {
+        *(f32x4*)p = v;
+      }
+    } else {
+      const u32x2 v = *(const u32x2*)((const uint16_t*)rows + h * D + d);
+      uint16_t* p = (uint16_t*)a.out + off;
+      if (through) {
+        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+      } else {
+        *(u32x2*)p = v;
+      }
+    }
+    if (d == 0 && !a.no_lse) {
+      const float lse = lse_slot[h];
+      if (a.lse) {
+        a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
+      } else {
+        store_partial1(a.out, off + D, a.mid_dtype, lse, through);
+      }
+    }
   }
 }
 

@@ -257,6 +257,30 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
     }
   };
   const int nheads = min(kHB, a.G - w.hb * kHB);
+  // Chunked work items: a finished split -> a parked slot as the finished partial (SplitArgs::park_final): fp32 LSEs,
+  // then normalised rows in mid_dtype, times the V scale.  A lane holds eight consecutive dims of head 16*nb + c per i.
+  auto park_final = [&](char* slot) {
+    wave_lds_fence();
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float lsum = l[nb];
+      lsum += __shfl_xor(lsum, 16);
+      lsum += __shfl_xor(lsum, 32);
+      const int h = 16 * nb + c;
+      if (h < nheads) {
+        const float inv = lsum > 0.f ? v_scale / lsum : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 4 * g + i;
+          float v[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[j] = acc[nb][j][i] * inv;
+          park_store8(slot + kHB * 4, h * kD + 16 * (r & 7) + 8 * (r >> 3), a.mid_dtype, v);
+        }
+        if (g == 0) ((float*)slot)[h] = lsum > 0.f ? (m[nb] + fd_log2(lsum)) * FD_LN2 : -INFINITY;
+      }
+    }
+  };
 
   if constexpr (CHUNK) {
     // Wave-uniform cursors over the tiles of the wave's splits (as in the 16-bit kernel): a tile starts at `base`
@@ -278,8 +302,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
     };
     // Finished partials other than the wave's last one wait in LDS behind the staging buffers (a.park slots per
     // wave); all of them are stored when the wave has issued its last load.
-    constexpr int kPartFloats = kHB * kD + 2 * kHB;
-    float* park = (float*)(smem + a.hpw * a.nsub * kWaveLds) + (size_t)(wave * a.park) * kPartFloats;
+    char* park = smem + a.hpw * a.nsub * kWaveLds + (size_t)(wave * a.park) * a.park_bytes;
     int parked = 0;
     bool last_staged = false;
     Cur cur{__builtin_amdgcn_readfirstlane(w.start), 0};
@@ -300,7 +323,11 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
       while (!(cur.end >= run_end && cur.base + kTile >= cur.end)) {   // all tiles but the wave's last one
         tile(cur.base, cur.end, lookup2, std::true_type{});
         if (cur.base + kTile >= cur.end) {   // that was the last tile of a split
-          stage_partial(park + parked * kPartFloats);
+          if (a.park_final) {
+            park_final(park + parked * a.park_bytes);
+          } else {
+            stage_partial((float*)(park + parked * a.park_bytes));
+          }
           ++parked;
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
@@ -320,7 +347,12 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
     wave_lds_fence();
     for (int i = 0; s_cur + i < s_lim; ++i) {   // splits beyond the sequence's end are stored as empty
       const bool empty = i > parked || (i == parked && !last_staged);
-      wave_store_partial<kHB, kD>(a, i < parked ? park + i * kPartFloats : part, w.b, head0, nheads, s_cur + i, empty);
+      if (i < parked && a.park_final) {
+        wave_copy_parked<kHB, kD>(a, park + i * a.park_bytes, w.b, head0, nheads, s_cur + i);
+      } else {
+        wave_store_partial<kHB, kD>(a, i < parked ? (const float*)(park + i * a.park_bytes) : part, w.b, head0, nheads,
+                                    s_cur + i, empty);
+      }
     }
   } else {
     if (t0 < t1) {
@@ -365,7 +397,7 @@ int fd_launch_split_mfma_fp8(hipStream_t stream, const SplitArgs& a, int q_dtype
   const unsigned block = 64u * waves;
   const int nb = a.hbsz > 16 ? 2 : 1;   // a.hbsz = query heads per head block: up to 16, or up to 32 (two per wave)
   size_t lds = (size_t)waves * wave_lds(nb);
-  if (a.chunk > 1) lds += (size_t)waves * a.park * (16 * nb * kD + 2 * 16 * nb) * 4;   // parked partials
+  if (a.chunk > 1) lds += (size_t)waves * a.park * a.park_bytes;   // parked partials
   if (a.tickets) {  // the fused combine stages (S + num_extra) LSEs per head in LDS
     const size_t need = (size_t)(a.S + a.num_extra) * 16 * nb * 4;
     if (need > lds) lds = need;
