@@ -6,7 +6,7 @@ import random
 import pytest
 import torch
 
-from helpers import assert_lse_close, assert_out_close, oracle_decode, run_decode
+from helpers import assert_lse_close, assert_out_close, assert_out_rel, oracle_decode, run_decode
 
 pytestmark = pytest.mark.gpu
 
@@ -113,3 +113,58 @@ def test_random_serving_shape(fd, i):
     out, lse = run_decode(fd, wl, variant=c["variant"], **kw)
     assert_out_close(out, ref, atol=2e-2)
     assert_lse_close(lse, ref_lse, rtol=1e-3)
+
+
+# ---- third sweep: exactly the caller's split count on head_dim 128 with sequences long enough for chunked work items
+# (a workgroup walks several splits, a wave parks finished or raw partials in LDS): internal partials and
+# caller-visible [B, Hq, S, D + 1] buffers of every element type, groups up to 32 query heads
+EXACT_CASES = 60
+
+
+def _exact_case(i):
+    rng = random.Random(21000 + i)
+    kind = rng.choice(["bf16", "fp16", "fp8"])
+    Hkv = rng.choice([1, 2, 4, 8])
+    G = rng.choice([1, 4, 4, 8, 8, 16, 20, 32])
+    B = rng.choice([1, 2, 3, 8, 9])
+    P = rng.choice([1, 16, 16, 64])
+    top = rng.choice([600, 3000, 9000])
+    lens = [rng.choice([0, 1, 63, 64, 65, 2047, 2048, 2049]) if rng.random() < 0.25 else rng.randint(1, top)
+            for _ in range(B)]
+    lens[0] = max(lens[0], top // 2)
+    return dict(kind=kind, Hq=Hkv * G, Hkv=Hkv, P=P, lens=lens, kv_split=rng.choice([2, 3, 7, 16, 24, 32, 64]),
+                soft_cap=rng.choice([0.0, 0.0, 30.0]), visible=rng.choice([None, None, "f32", "bf16", "f16"]),
+                offset=rng.random() < 0.3)
+
+
+@pytest.mark.parametrize("i", range(EXACT_CASES))
+def test_random_exact_split_shape(fd, i):
+    c = _exact_case(i)
+    D = 128
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp8": torch.bfloat16}[c["kind"]]
+    wl = fd.utils.make_paged_workload(f"exact{i}", c["lens"], c["Hq"], c["Hkv"], D, c["P"], dtype, c["kv_split"],
+                                      seed=23000 + i, soft_cap=c["soft_cap"], fp8_kv=c["kind"] == "fp8")
+    ref, ref_lse = oracle_decode(wl)
+    kw, mid = {}, None
+    lse_rtol, rms_rtol, max_rtol = 1e-3, 1e-2, 2e-2
+    if c["visible"] is None:
+        kw["plan_splits"] = False
+    else:
+        mdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[c["visible"]]
+        B, S = len(c["lens"]), c["kv_split"]
+        n = B * c["Hq"] * S * (D + 1)
+        flat = torch.full((n + 1,), float("nan"), dtype=mdt, device="cuda:0")
+        # (some buffers start one element past an aligned address)
+        mid = (flat[1:] if c["offset"] else flat[:n]).view(B, c["Hq"], S, D + 1)
+        kw["output_split"] = mid
+        if mdt != torch.float32:
+            lse_rtol = 1e-2   # the partial LSEs are held in 16 bits as well ...
+        if mdt == torch.bfloat16:
+            # ... in bf16 with 8 bits of mantissa: an LSE near 9 is off by up to 0.02, and so are the merge weights
+            rms_rtol, max_rtol = 3e-2, 6e-2
+    out, lse = run_decode(fd, wl, **kw)
+    if mid is not None:
+        assert not torch.isnan(mid).any(), "a partial slot was not written"
+    assert_out_close(out, ref, atol=2e-2, rel=False)
+    assert_out_rel(out, ref, rms_rtol=rms_rtol, max_rtol=max_rtol)
+    assert_lse_close(lse, ref_lse, rtol=lse_rtol)
