@@ -123,9 +123,11 @@ typedef struct fd_params {
   int32_t v_head_dim;       /* 0: Dv = head_dim.  Else 64, 128 or 256: the V cache's head dim, which the
                                reference takes from the V cache independently of K's (V_DIM next to K_DIM,
                                flash_decode.py:162-163, 765-774).  Partials and outputs then have Dv (+1)
-                               columns and fd_combine works on Dv.  Dv != Dk runs on the VALU kernel
-                               (fp32 / fp16 / bf16 caches; FD_ERR_UNSUPPORTED with FD_PATH_MFMA, with an
-                               fp8 cache and in fd_kv_append).                                  */
+                               columns and fd_combine works on Dv.  Dv != Dk: fp32 / fp16 / bf16 caches.
+                               A K head dim of 128 with a V head dim of 64 or 256, a 16-bit cache and up
+                               to 16 query heads per KV head runs on the MFMA kernel, everything else on
+                               the VALU kernel (FD_ERR_UNSUPPORTED for the other shapes with
+                               FD_PATH_MFMA, with an fp8 cache and in fd_kv_append).            */
 } fd_params;
 
 /*

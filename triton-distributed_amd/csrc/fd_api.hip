@@ -300,14 +300,21 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
 
   const bool q16 = p->q_dtype == FD_BF16 || p->q_dtype == FD_F16;
   const bool kv_fp8 = p->kv_dtype == FD_FP8_E4M3;
-  const bool mfma_ok = mfma_shape_ok(D, p->kv_dtype) && Dv == D && q16 && (kv_fp8 || p->q_dtype == p->kv_dtype) &&
-                       aligned16(q) && stride_q_bs % 8 == 0 && stride_q_h % 8 == 0;
+  // V head dim 64 or 256 beside a K head dim of 128: the head_dim-128 16-bit kernel with its V side narrowed or split
+  // into two members (groups of up to 16 query heads, two launches)
+  const bool fuse_wanted = tail && tail->tickets && p->mid_dtype == FD_F32;
+  const bool dv_mfma = Dv != D && D == 128 && !kv_fp8 && (Dv == 64 || Dv == 256) && G <= 16 && !fuse_wanted &&
+                       stride_v_h % 8 == 0 && stride_v_tok % 8 == 0;
+  const bool mfma_ok = mfma_shape_ok(D, p->kv_dtype) && (Dv == D || dv_mfma) && q16 &&
+                       (kv_fp8 || p->q_dtype == p->kv_dtype) && aligned16(q) && stride_q_bs % 8 == 0 &&
+                       stride_q_h % 8 == 0;
   bool use_mfma = mfma_ok;
   if (p->path == FD_PATH_VALU) use_mfma = false;
   if (p->path == FD_PATH_MFMA && !mfma_ok)
     return fail(FD_ERR_UNSUPPORTED,
                 "%s: MFMA path needs a 16-bit query with a KV cache of the same dtype or fp8-e4m3, equal K and V head "
-                "dims and 16-byte aligned q rows", fn);
+                "dims (or K 128 with V 64 / 256, 16-bit cache, up to 16 query heads per KV head, no fused combine) and "
+                "16-byte aligned q rows", fn);
   if (p->waves_per_block != 0 && p->waves_per_block != 1 && p->waves_per_block != 2 && p->waves_per_block != 4 &&
       p->waves_per_block != 8)
     return fail(FD_ERR_INVALID_ARG, "%s: waves_per_block %d (0, 1, 2, 4 or 8)", fn, p->waves_per_block);
@@ -341,7 +348,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   int chunk_wish = 1;
   // Not for large batches: their lengths differ in practice, and many short work items balance better over the CUs
   // than few long ones (config 4's ragged batch of 64 with exactly 32 splits: 691 us unchunked, 713 us chunked).
-  if (use_mfma && D == 128 && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
+  if (use_mfma && D == 128 && Dv == D && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
       batch <= kMaxChunkBatch && !env_no_chunk()) {
     fd_params plan = *p;
     plan.split_adapt = 0;
@@ -396,6 +403,23 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   } else if (use_mfma && !fuse) {
     a.hpw = choose_heads_per_group(a.Hkv, D * kvsz * (pair ? 2 : 1), waves, wgs, max_waves);
   }
+  // V head dim: the column of an in-row LSE; on the head_dim-128 MFMA kernel a V head dim of 256 makes every KV head
+  // two workgroup members (one per 128-column half), one of 64 narrows the V fetch and the stored columns
+  a.dv = Dv;
+  a.v_members = 1;
+  a.v_chunk_mask = 15;
+  a.v_cols = 1 << 30;
+  if (use_mfma && Dv != D) {
+    if (Dv == 256) {
+      while (waves * 2 > max_waves) waves >>= 1;
+      const int heads = choose_heads_per_group(a.Hkv, D * kvsz, waves * 2, wgs, max_waves);
+      a.v_members = 2;
+      a.hpw = 2 * heads;
+    } else {
+      a.v_chunk_mask = 7;
+      a.v_cols = 64;
+    }
+  }
   if (a.chunk > 1) {
     // two chunked workgroups per CU: fewer parked splits per wave if their LDS would not allow it
     const int wave_lds = hb_slots_lds(a.hbsz);
@@ -405,7 +429,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     a.chunk = waves * chunk_per_wave;
     a.park = chunk_per_wave - 1;
   }
-  a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / a.hpw * a.nhb;
+  a.grid_x = a.member_hb ? a.Hkv * (a.nhb / a.hpw) : a.Hkv / (a.hpw / a.v_members) * a.nhb;
   a.nsub = waves;
   waves *= a.hpw;   // total waves of a workgroup
 
@@ -572,7 +596,9 @@ static int64_t plan_fill_splits(const char* fn, const fd_params* p, int32_t batc
       p->page_size <= 0 || p->max_pages_per_seq <= 0)
     return fail(FD_ERR_INVALID_ARG, "%s: batch, heads, num_splits, page_size, max_pages_per_seq must be > 0", fn);
   const int G = p->q_heads / p->kv_heads;
-  const bool mfma = mfma_shape_ok(p->head_dim, p->kv_dtype) && v_dim(p) == p->head_dim && p->path != FD_PATH_VALU;
+  const bool dv_mfma = p->head_dim == 128 && p->kv_dtype != FD_FP8_E4M3 && (v_dim(p) == 64 || v_dim(p) == 256) && G <= 16;
+  const bool mfma = mfma_shape_ok(p->head_dim, p->kv_dtype) && (v_dim(p) == p->head_dim || dv_mfma) &&
+                    p->path != FD_PATH_VALU;
   const int hb = mfma ? mfma_head_block(p->head_dim, G, p->kv_dtype) : (G >= 3 ? 4 : G);
   const int64_t nhb = (G + hb - 1) / hb;
   // fp8 rows of head_dim 64: two KV heads per wave (the usual cache layout has their rows side by side)

@@ -66,6 +66,11 @@ struct SplitArgs {
   int32_t store_through;          // 1: partials are written through to memory (sc0 sc1) instead of being left dirty in
                                   // the XCD's L2 until the kernel ends; pays off for tens of MB of partials
   int32_t park;                   // chunked work items: finished partials a wave parks in LDS besides its last one
+  // V head dim != K head dim on the head_dim-128 MFMA kernel.  dv = V head dim (the column of an in-row LSE).
+  // v_members = 2 (dv 256): a workgroup member is a (KV head, 128-column half of the V rows) pair -- two waves share
+  // K and the softmax and each accumulates and stores its own half.  v_chunk_mask = 7 (dv 64): the 16 lanes of a
+  // wave row fetch the eight 16-byte chunks of a 128-byte V row twice, and only v_cols = 64 columns are stored.
+  int32_t dv, v_members, v_chunk_mask, v_cols;
   int32_t park_final;             // 1: a parked partial is the finished one -- fp32 LSEs of the wave's head slots, then
                                   // normalised rows [head][D] in mid_dtype (rows that start on multiples of four
                                   // elements only); 0: the wave's raw state in cta_merge_store's layout
@@ -323,6 +328,7 @@ __device__ __forceinline__ int tokens_per_range(int kv_len, int S, uint32_t s_ma
 struct WorkItem {
   int b, s, kvh, hb, start, end;
   bool skip;  // empty range and nothing to write: the workgroup may leave at once (uniform over the workgroup)
+  int vh;     // 128-column half of the V rows this wave accumulates (SplitArgs::v_members == 2), else 0
   int kvh0;   // first KV head of the workgroup
   int hb0;    // first head block of the workgroup
   int sub;    // token sub-range index of this wave
@@ -334,6 +340,7 @@ struct WorkItem {
 
 __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   WorkItem w;
+  w.vh = 0;
   // The sequence and its length first: these scalar loads head the chain length -> block table -> K/V rows that
   // every wave has to walk before it can stream.
   int b, s;
@@ -383,6 +390,12 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
       w.kvh0 = grp;
       w.kvh = grp;
       w.sub = wave;
+    } else if (a.v_members == 2) {   // members are (KV head, V half) pairs: hpw / 2 heads per workgroup
+      const int member = wave - (wave / a.hpw) * a.hpw;
+      w.kvh0 = grp * (a.hpw >> 1);
+      w.sub = wave / a.hpw;
+      w.kvh = w.kvh0 + (member >> 1);
+      w.vh = member & 1;
     } else {
       w.kvh0 = grp * a.hpw;
       w.sub = wave / a.hpw;
@@ -522,13 +535,14 @@ __device__ __forceinline__ void cta_merge_store_rounds(const SplitArgs& a, float
       default: weigh(std::integral_constant<int, 0>{}, w.nsub);
     }
     ml[HB] = L > 0.f ? 1.0f / L : 0.f;
-    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + (a.v_members == 2 ? hm >> 1 : hm);
+    const int co = a.v_members == 2 ? (hm & 1) * 128 : 0;   // this member's half of the V columns
     const int hb = a.member_hb ? w.hb0 + hm : w.hb;
-    if (h < a.G - hb * HB && (a.tickets || !a.no_lse)) {
+    if (h < a.G - hb * HB && co == 0 && (a.tickets || !a.no_lse)) {
       const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
       const int head = kvh * a.G + hb * HB + h;
       const int64_t lse_at = ((int64_t)w.b * a.Hq + head) * a.S + w.s;
-      const int64_t col_d = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + D;
+      const int64_t col_d = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + a.dv;
       if (a.tickets) {   // fused combine (fp32 partials only): another XCD's workgroup may read these
         store_f32_agent(a.lse ? a.lse + lse_at : (float*)a.out + col_d, lse);
       } else if (a.lse) {
@@ -561,9 +575,10 @@ __device__ __forceinline__ void cta_merge_store_rounds(const SplitArgs& a, float
       const int r = e - hm * per_member;
       const int h = r / PER_ROW;
       const int d = (r - h * PER_ROW) * V;
-      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + (a.v_members == 2 ? hm >> 1 : hm);
+      const int co = a.v_members == 2 ? (hm & 1) * 128 : 0;   // this member's half of the V columns
       const int hb = a.member_hb ? w.hb0 + hm : w.hb;
-      if (h >= a.G - hb * HB) continue;
+      if (h >= a.G - hb * HB || d >= a.v_cols) continue;
       const float* x0 = part + hm * stride + h * D + d;
       const float* w0 = part + hm * stride + HB * D + h;
       Val o{};
@@ -583,7 +598,7 @@ __device__ __forceinline__ void cta_merge_store_rounds(const SplitArgs& a, float
       }
       o *= inv;
       const int head = kvh * a.G + hb * HB + h;
-      const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;
+      const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d + co;
       if constexpr (V == 4) {
         if (fused) {
 #pragma unroll
@@ -628,9 +643,10 @@ __device__ __forceinline__ void cta_merge_store_one_round(const SplitArgs& a, co
       const int r = e - hm * heads * D;
       const int h = r / D;
       const int d = r - h * D;
-      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+      const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + (a.v_members == 2 ? hm >> 1 : hm);
+      const int co = a.v_members == 2 ? (hm & 1) * 128 : 0;   // this member's half of the V columns
       const int hb = a.member_hb ? w.hb0 + hm : w.hb;
-      if (h >= a.G - hb * HB) continue;
+      if (h >= a.G - hb * HB || d >= a.v_cols) continue;
       float M = -INFINITY;
       for (int p = 0; p < w.nsub; ++p) M = fmaxf(M, part[(hm + a.hpw * p) * stride + HB * D + h]);
       float L = 0.f, o = 0.f;
@@ -645,13 +661,13 @@ __device__ __forceinline__ void cta_merge_store_one_round(const SplitArgs& a, co
       const float inv = L > 0.f ? 1.0f / L : 0.f;
       const int head = kvh * a.G + hb * HB + h;
       const int64_t row = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s;
-      store_partial1(a.out, row + d, a.mid_dtype, o * inv, a.store_through != 0);
-      if (d == 0 && !a.no_lse) {
+      store_partial1(a.out, row + d + co, a.mid_dtype, o * inv, a.store_through != 0);
+      if (d == 0 && co == 0 && !a.no_lse) {
         const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
         if (a.lse) {
           a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
         } else {
-          store_partial1(a.out, row + D, a.mid_dtype, lse, a.store_through != 0);
+          store_partial1(a.out, row + a.dv, a.mid_dtype, lse, a.store_through != 0);
         }
       }
     }
@@ -667,9 +683,10 @@ __device__ __forceinline__ void cta_merge_store_one_round(const SplitArgs& a, co
     }
     const int h = r / D4;
     const int d = (r - h * D4) * 4;
-    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + hm;
+    const int kvh = a.member_hb ? w.kvh0 : w.kvh0 + (a.v_members == 2 ? hm >> 1 : hm);
+    const int co = a.v_members == 2 ? (hm & 1) * 128 : 0;   // this member's half of the V columns
     const int hb = a.member_hb ? w.hb0 + hm : w.hb;
-    if (h >= a.G - hb * HB) continue;
+    if (h >= a.G - hb * HB || d >= a.v_cols) continue;
     // This runs once per workgroup, after the last tile, with nothing left to overlap: every LDS read below is
     // requested before the first one is used (unrolled over the sub-ranges; a loop over a run-time count takes one
     // dependent LDS round trip per sub-range and value, about 1 us per launch in all).
@@ -716,24 +733,26 @@ __device__ __forceinline__ void cta_merge_store_one_round(const SplitArgs& a, co
     float inv = L > 0.f ? 1.0f / L : 0.f;
     o *= inv;
     const int head = kvh * a.G + hb * HB + h;
-    const int64_t off = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s + d;
+    const int64_t row = (int64_t)w.b * a.so_b + (int64_t)head * a.so_h + (int64_t)w.s * a.so_s;
+    const int64_t off = row + d + co;
     const float lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
     if (a.tickets) {
       // fused combine (fp32 partials only): another XCD's workgroup may read these
 #pragma unroll
       for (int i = 0; i < 4; ++i) store_f32_agent((float*)a.out + off + i, o[i]);
-      if (d == 0) store_f32_agent(a.lse ? a.lse + ((int64_t)w.b * a.Hq + head) * a.S + w.s : (float*)a.out + off + D, lse);
+      if (d == 0 && co == 0)
+        store_f32_agent(a.lse ? a.lse + ((int64_t)w.b * a.Hq + head) * a.S + w.s : (float*)a.out + row + a.dv, lse);
     } else {
       if (a.vec_out) {
         store_partial4(a.out, off, a.mid_dtype, o, a.store_through != 0);
       } else {
         for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
       }
-      if (d == 0 && !a.no_lse) {
+      if (d == 0 && co == 0 && !a.no_lse) {
         if (a.lse) {
           a.lse[((int64_t)w.b * a.Hq + head) * a.S + w.s] = lse;
         } else {
-          store_from_f32(a.out, off + D, a.mid_dtype, lse);
+          store_from_f32(a.out, row + a.dv, a.mid_dtype, lse);
         }
       }
     }

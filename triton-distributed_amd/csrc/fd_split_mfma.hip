@@ -91,7 +91,8 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
 
   const int32_t* bt_row = a.bt + (int64_t)w.b * a.sbt;
   const char* kbase = (const char*)a.k + ((int64_t)w.kvh * a.sk_h) * 2 + c * 16;
-  const char* vbase = (const char*)a.v + ((int64_t)w.kvh * a.sv_h) * 2 + c * 16;
+  // (V head dim 64: the 16 lanes of a wave row fetch the 8 chunks of a 128-byte row twice; 256: this wave's half)
+  const char* vbase = (const char*)a.v + ((int64_t)w.kvh * a.sv_h) * 2 + (c & a.v_chunk_mask) * 16 + w.vh * 256;
   const int k_pitch = (int)(a.sk_t * 2);
   const int v_pitch = (int)(a.sv_t * 2);
   char* kb = smem + wave * kWaveLds;
