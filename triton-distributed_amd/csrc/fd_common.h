@@ -765,7 +765,8 @@ template <int HB, int D>
 __device__ __forceinline__ void cta_merge_store(const SplitArgs& a, float* part, int stride, const WorkItem& w,
                                                 int nheads) {
   const int heads = a.member_hb ? HB : nheads;
-  if (a.hpw * heads * (D / 4) <= 2 * 64 * a.hpw * a.nsub) {
+  const bool by_element = !a.vec_out && !a.tickets;   // one value per thread and round: four times the rounds
+  if (a.hpw * heads * (D / 4) <= 2 * 64 * a.hpw * a.nsub && !by_element) {
     cta_merge_store_one_round<HB, D>(a, part, stride, w, nheads);
   } else {
     cta_merge_store_rounds<HB, D>(a, part, stride, w, nheads);
