@@ -134,7 +134,7 @@ def _exact_case(i):
     lens[0] = max(lens[0], top // 2)
     return dict(kind=kind, Hq=Hkv * G, Hkv=Hkv, P=P, lens=lens, kv_split=rng.choice([2, 3, 7, 16, 24, 32, 64]),
                 soft_cap=rng.choice([0.0, 0.0, 30.0]), visible=rng.choice([None, None, "f32", "bf16", "f16"]),
-                offset=rng.random() < 0.3)
+                offset=rng.random() < 0.3, variant=rng.choice(["plain", "plain", "persistent"]))
 
 
 @pytest.mark.parametrize("i", range(EXACT_CASES))
@@ -162,7 +162,7 @@ def test_random_exact_split_shape(fd, i):
         if mdt == torch.bfloat16:
             # ... in bf16 with 8 bits of mantissa: an LSE near 9 is off by up to 0.02, and so are the merge weights
             rms_rtol, max_rtol = 3e-2, 6e-2
-    out, lse = run_decode(fd, wl, **kw)
+    out, lse = run_decode(fd, wl, variant=c["variant"], **kw)   # persistent: (sequence, range) items in issue order
     if mid is not None:
         assert not torch.isnan(mid).any(), "a partial slot was not written"
     assert_out_close(out, ref, atol=2e-2, rel=False)

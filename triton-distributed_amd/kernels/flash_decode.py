@@ -284,8 +284,9 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
         assert seq_order_lens.numel() == batch
     # Work-item order ((sequence, range) items, largest first, empty ranges last): given by the caller (the append
-    # launch computed it) or computed here by one scheduling launch.  Internal partials and planned splits only.
-    want_items = (item_order is not None or schedule_items) and split_adapt > 0 and num_splits > 1 and not fuse_combine
+    # launch computed it) or computed here by one scheduling launch.  With the caller's exact split count the items are
+    # the reference's ranges (every slot of the partial buffer is still written, empty ranges last).
+    want_items = (item_order is not None or schedule_items) and num_splits > 1 and not fuse_combine
     if want_items and item_order is None and batch > MAX_ITEM_BATCH:
         want_items = False
     if schedule_items and not want_items and seq_order is None and num_splits > 1 and batch <= MAX_ITEM_BATCH:
