@@ -94,13 +94,19 @@ def make_pools(torch, wl, dev, n):
     return pools
 
 
+def _flash_decode(fd):
+    return importlib.import_module(fd.__name__ + ".kernels.flash_decode")
+
+
 def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="auto", waves=0, fuse=False):
     """The decode step of a workload as a callable of the step index, plus its output and LSE tensors."""
     B, Hq, D = wl.q.shape
     out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
     # kv_split -1: the library chooses the split count and owns the partials
-    workspace = torch.empty(B * Hq * S * (D + 1), dtype=torch.float32, device=dev) if S > 0 else None
+    # room for the partials of as many splits as the step may be planned with
+    S_ws = max(S, 0) if exact else _flash_decode(fd).split_bound(S, wl.block_table.shape[1] * wl.k_cache.shape[1])
+    workspace = torch.empty(B * Hq * S_ws * (D + 1), dtype=torch.float32, device=dev) if S_ws > 0 else None
     q_lens = [1] * B
     kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=path, waves_per_block=waves, fuse_combine=fuse)
     if wl.k_scale is not None:
@@ -163,7 +169,7 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     """Every north-star figure besides the headline, in this same process, each as (microseconds per decode step,
     fraction of the 8 TB/s peak on the step's algorithmic bytes): config 2 with exactly the 32 splits the workload
     names; config 5 (fp8 KV) and its bf16 twin, planned and with exactly 64 splits, and their ratios (target >= 1.7);
-    config 3; config 4 scheduled and unscheduled."""
+    config 3, planned and with exactly 32 splits; config 4 scheduled and unscheduled."""
     U = fd.utils
     t = {}
     # the headline times exactly the steps the command line asks for; these side figures take at least 100 steps and
@@ -187,6 +193,7 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     del c5, c5t
     c3 = U.make_config(3)
     put("c3_sp_shard_plus_7_partials", measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0))
+    put("c3_exact_32_splits", measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0, exact=True))
     del c3
     c4 = U.make_config(4)
     n4 = steps // 4   # a step of config 4 is 15 times config 2's
@@ -383,9 +390,8 @@ def main():
     lib = fd.load_library()
     fk = importlib.import_module("triton-distributed_amd.kernels.flash_decode")
     S_bound = S
-    if S == -1:   # the library's own bound, as in the wrapper
-        capacity = wl.block_table.shape[1] * wl.k_cache.shape[1]
-        S_bound = fk.auto_split_bound(capacity)
+    if not args.exact_splits:   # the library's own bound, as in the wrapper (the caller's count is a hint there)
+        S_bound = fk.split_bound(S, wl.block_table.shape[1] * wl.k_cache.shape[1])
     p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_bound, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
                         wl.k_scale, wl.v_scale, args.path, args.waves)
     p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials
