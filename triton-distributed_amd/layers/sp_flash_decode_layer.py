@@ -17,7 +17,7 @@ Step 2 is where the reference allgathers over NVSHMEM (:139).  Nothing here
 spans more than one GPU: the other ranks' slots are filled from
 ``remote_partials`` -- ``(out [R-1, B, Hq, Dv], lse [R-1, B, Hq])`` in rank order
 with this rank left out -- which the caller produces on the same device.  With
-``num_ranks == 1`` no remote partials are needed.  The staged slots keep the
+``num_ranks == 1`` no remote partials are needed and steps 2 and 3 fall away: the local decode writes the final output.  The staged slots keep the
 layout a push-allgather would write into, so one can be put in front of step 3
 later without touching the kernels.
 
@@ -31,7 +31,8 @@ from typing import Optional, Tuple
 
 import torch
 
-from ..kernels.flash_decode import (gqa_fwd_batch_decode_intra_rank, kernel_inter_rank_gqa_fwd_batch_decode_combine_kv)
+from ..kernels.flash_decode import (gqa_fwd_batch_decode, gqa_fwd_batch_decode_intra_rank,
+                                    kernel_inter_rank_gqa_fwd_batch_decode_combine_kv)
 
 
 class SpGQAFlashDecodeAttention(torch.nn.Module):
@@ -110,6 +111,16 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         if self.num_ranks > 1 and remote_partials is None:
             raise RuntimeError(
                 "num_ranks > 1 needs remote_partials: this build runs on one GPU and performs no allgather")
+
+        if self.num_ranks == 1:
+            # nothing to merge across ranks: the local decode writes the final output itself (split + combine, no
+            # staging and no third launch); the ring position still advances once per call
+            final_output = torch.empty([batch, self.num_q_heads, self.v_head_dim], dtype=q.dtype, device=q.device)
+            gqa_fwd_batch_decode(q, k_cache, v_cache, self.workspace, [1] * batch, global_kv_lens[0], block_table,
+                                 self.scale, soft_cap=self.soft_cap, output_split=output_split,
+                                 output_combine=final_output, kv_split=self.kv_split)
+            self.signal_target += 1
+            return final_output
 
         pdtype = self.partial_dtype or q.dtype
         d1 = self.v_head_dim + 1
