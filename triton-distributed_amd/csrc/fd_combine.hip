@@ -149,12 +149,26 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   *(f32x4*)&s_acc[tid * 4] = acc;   // row r, columns 4 * (tid % CG) .. + 3 of the chunk
   if ((tid & (CG - 1)) == 0) s_l[r] = L;
   __syncthreads();
-  if (tid < 4 * CG) {
-    float o = 0.f, Lsum = 0.f;
-    for (int i = 0; i < ROWS; ++i) {
-      o += s_acc[i * 4 * CG + tid];
-      Lsum += s_l[i];
-    }
+  // Sum over the ROWS row groups in two short steps instead of one thread per column walking all of them (64 dependent
+  // LDS reads for a 16-column chunk): thread (g, col) adds the four rows g, g + NG, g + 2 NG, g + 3 NG of its column
+  // (ROWS = 4 NG), the NG sums of a column go back through LDS, and the sum of the weights is a butterfly over one wave.
+  const int ncol = 4 * CG;
+  const int NG = kCombineThreads / ncol;        // = ROWS / 4
+  const int col = tid & (ncol - 1);
+  const int g = tid >> (a.cg_shift + 2);
+  float part4 = 0.f;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) part4 += s_acc[(g + k * NG) * ncol + col];
+  float lw = (tid & 63) < ROWS ? s_l[tid & 63] : 0.f;   // ROWS <= 64
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) lw += __shfl_xor(lw, off);
+  __syncthreads();
+  s_acc[g * ncol + col] = part4;
+  __syncthreads();
+  if (tid < ncol) {
+    float o = 0.f;
+    for (int i = 0; i < NG; ++i) o += s_acc[i * ncol + tid];
+    const float Lsum = lw;
     const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
     const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
     store_from_f32(a.out, out_base + col0 + tid, a.out_dtype, o * inv);
