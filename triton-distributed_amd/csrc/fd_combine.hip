@@ -232,9 +232,13 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
     }
   }
   float mine = -INFINITY;   // LSE of partial `lane`: from its own buffer, or from column D of the partial's row
-  if (lane < S)
+  if (lane < S) {
     mine = a.mid_lse ? a.mid_lse[((int64_t)b * a.Hq + h) * S + lane]
                      : load_as_f32(a.mid_o, mid_base + (int64_t)lane * a.s_ms + D, MID);
+    // partials of other ranks: rank `lane` counts iff it holds tokens of this sequence (flash_decode.py:513-515);
+    // what its slot holds otherwise is not looked at (the rows are requested, their values dropped below)
+    if (a.mode == FD_COMBINE_RANK && a.seqlens[(int64_t)lane * a.batch + b] <= 0) mine = -INFINITY;
+  }
   float M = mine;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
@@ -245,7 +249,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
     const int s = r + p * ROWS;
     const float own = __shfl(mine, s & 63);          // -inf for empty and absent splits: weight 0
     const float wgt = M > -INFINITY && s < S ? __expf(own - M) : 0.f;
-    acc += o[p] * wgt;
+    if (wgt != 0.f) acc += o[p] * wgt;   // (a slot that does not count may hold anything, NaN included)
     L += wgt;
   }
   if constexpr (VEC) {
@@ -320,11 +324,12 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   CombineArgs a = args;
   const int64_t rows = (int64_t)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
-  // the short kernel: this library's own partials in the same call, all slots written, at most 64 of them -- above
+  // the short kernel: this library's own partials in the same call (all slots written) or the per-rank partials of the
+  // inter-rank merge (validity by the ranks' lengths), at most 64 of them -- above
   // 32 only where there is a workgroup per CU: with few output rows (one long sequence: 96 rows x 42 partials) the
   // general kernel, which spreads a row over several workgroups, is the faster one (5.0 against 5.7 us)
   const int np_own = a.num_partials <= 16 ? 16 : (a.num_partials <= 32 ? 32 : 64);
-  const bool small = a.all_slots_written && a.mode != FD_COMBINE_RANK && a.num_extra == 0 &&
+  const bool small = (a.all_slots_written || a.mode == FD_COMBINE_RANK) && a.num_extra == 0 &&
                      (a.num_partials <= 32 || (a.num_partials <= 64 && rows >= 256));
   // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
   // one workgroup per CU and a thread would still have more than two partials to walk.
