@@ -1,6 +1,6 @@
 /*
  * A consumer of the C ABI with no Python in the loop: fills a small paged decode problem, runs fd_decode (and
- * fd_schedule, fd_plan_splits, fd_kv_append) from libflash_decode_gfx950.so on the GPU and checks the result
+ * fd_decode_noalloc, fd_schedule, fd_plan_splits, fd_kv_append) from libflash_decode_gfx950.so on the GPU and checks the result
  * against the plain-C oracle (oracle/c/ref_decode.c).  Exit code 0 = all checks passed.
  *
  *   gcc -O2 -std=c11 -D__HIP_PLATFORM_AMD__ tests/c_abi/run_c_abi.c oracle/c/ref_decode.c -Iinclude -I/opt/rocm/include \
@@ -116,6 +116,22 @@ int main(void) {
     if (!(fabs((double)lse[i] - (double)ref_lse[i]) <= 1e-5 * fmax(1.0, fabs((double)ref_lse[i])))) ++bad;
   }
   printf("fd_decode (fp32, soft cap, scheduled, %d planned of %d splits): max |out - ref| = %.3e\n", planned, S, worst);
+
+  /* the entry point that allocates nothing (partials in the library's static device array): the same bits */
+  void *dout2 = NULL, *dlse2 = NULL;
+  HIP_OK(hipMalloc(&dout2, nq * 4));
+  HIP_OK(hipMalloc(&dlse2, sizeof(ref_lse)));
+  FD_OK_OR_DIE(fd_decode_noalloc(NULL, dq, dk, dv, dout2, (float*)dlse2, scale, (const int32_t*)dbt, (const int32_t*)dlens, B,
+                                 (int64_t)HQ * D, D, (int64_t)HKV * D, D, (int64_t)HKV * D, D, MAXP, (int64_t)HQ * D, D,
+                                 (const int32_t*)dorder, FD_COMBINE_SPLIT, NULL, NULL, 0, &p));
+  HIP_OK(hipDeviceSynchronize());
+  float* out2 = (float*)malloc(nq * 4);
+  float lse2[B * HQ];
+  HIP_OK(hipMemcpy(out2, dout2, nq * 4, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(lse2, dlse2, sizeof(lse2), hipMemcpyDeviceToHost));
+  if (memcmp(out, out2, nq * 4) != 0 || memcmp(lse, lse2, sizeof(lse)) != 0) { fprintf(stderr, "fd_decode_noalloc differs from fd_decode\n"); ++bad; }
+  if (fd_build_id() == NULL || strlen(fd_build_id()) == 0) { fprintf(stderr, "fd_build_id is empty\n"); ++bad; }
+  printf("fd_decode_noalloc: bit-identical to fd_decode = %s; library build id %s\n", bad ? "no" : "yes", fd_build_id());
 
   /* the write side: append one token per sequence (fp32 -> fp32 is a copy) and read it back */
   float knew[B * HKV * D], vnew[B * HKV * D];
