@@ -430,6 +430,8 @@ def main():
             wl.q.stride(0), wl.q.stride(1), k.stride(-3), k.stride(-2), v.stride(-3), v.stride(-2),
             mid.stride(0), mid.stride(1), mid.stride(2), wl.block_table.stride(0), order_ptr, byref(p)))
 
+    # (the graph capture above left the device idle for a few milliseconds: back to steady clocks first)
+    settle(torch, split_only, min(args.clock_ramp_ms, 50.0))
     for i in range(args.warmup):
         split_only(i)
     torch.cuda.synchronize()
