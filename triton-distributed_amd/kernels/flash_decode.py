@@ -27,14 +27,18 @@ Keyword-only additions that the reference does not have (all default off):
                   16 MiB of them) and the call allocates nothing -- for steps captured into a HIP graph or run where
                   allocation is not allowed; needs ``output_combine``; calls that overlap on one GPU must not share it
   fuse_combine    True: one launch, the combine runs in the tail of the split kernel (pays off when
-                  the groups of a ragged batch finish at different times); False (default): split
-                  kernel and combine kernel as two launches
+                  the groups of a ragged batch finish at different times, or for very short steps launched
+                  eagerly, where the second launch's host time counts); False (default): split kernel and
+                  combine kernel as two launches
 
 Differences from the reference, on purpose: when ``output_split`` is not
-supplied the partials are kept in fp32 with the LSE in its own fp32 buffer (the
-reference allocates fp16 ``[B,Hq,S,Dv+1]``, :783-784); the default
-``output_combine`` has the query's dtype (the reference hard-codes fp16, :785,
-which is the same thing for the fp16 inputs its tests use).
+supplied the partials stay inside the library as ``[B,Hq,S,Dv]`` with the LSEs
+in their own fp32 buffer -- fp32 values, or the output's 16-bit type once there
+are 4 MB of them or the caller insists on exactly ``kv_split`` splits
+(``internal_partial_dtype``; the reference allocates fp16 ``[B,Hq,S,Dv+1]``,
+:783-784); the default ``output_combine`` has the query's dtype (the reference
+hard-codes fp16, :785, which is the same thing for the fp16 inputs its tests
+use).
 """
 from __future__ import annotations
 
