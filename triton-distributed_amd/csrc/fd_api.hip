@@ -340,51 +340,74 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   if ((int64_t)a.Hkv * a.nhb >= ((int64_t)1 << 31))
     return fail(FD_ERR_TOO_LARGE, "%s: %lld workgroups per split", fn, (long long)a.Hkv * a.nhb);
   const bool fuse = tail && tail->tickets && p->mid_dtype == FD_F32;
-  // Chunked work items: the caller's split count and ranges are kept exactly (they are observable in out_split), but a
-  // workgroup walks `chunk` consecutive splits, so that the chip sees as many work items as the library's own plan
-  // would launch: every work item pays the prologue (arguments -> length -> block table -> first rows) once, not once
-  // per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.
-  a.chunk = 1;
-  int chunk_wish = 1;
-  // Not for large batches: their lengths differ in practice, and many short work items balance better over the CUs
-  // than few long ones (config 4's ragged batch of 64 with exactly 32 splits: 691 us unchunked, 713 us chunked).
-  if (use_mfma && D == 128 && Dv == D && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
-      batch <= kMaxChunkBatch && !env_no_chunk()) {
-    fd_params plan = *p;
-    plan.split_adapt = 0;
-    const int s_plan = fd_plan_splits(&plan, batch);
-    if (s_plan > 0 && s_plan < a.S) chunk_wish = (a.S + s_plan - 1) / s_plan;
-  }
-  a.chunk = chunk_wish;
-  const int items = (a.S + a.chunk - 1) / a.chunk;   // work items per (sequence, KV head, head block)
-  max_tok_split *= a.chunk;
-  // Ranges that are certain to be busy per sequence: all of them, or, when the ranges follow each sequence's own
-  // length, only the ones every sequence gets (the rest of the grid may be empty ranges).
-  const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : items;
-  const int64_t wgs = (int64_t)batch * busy_splits * a.Hkv * a.nhb;
   // the two-block MFMA kernel needs the register file of a whole SIMD per wave: workgroups of at most 4 waves
   const int max_waves = use_mfma && (a.hbsz > 16 || pair) ? 4 : 8;
   // the fp8 head_dim-64 kernel keeps 8 KB in flight per wave with one KV head per wave, like the VALU kernel;
   // the other MFMA kernels 16 KB
   const int64_t wave_target = use_mfma && !(kv_fp8 && D == 64 && !pair) ? kTargetWaves : kTargetWavesValu;
-  int waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
-                                 : choose_waves(wgs, max_tok_split, tile, wave_target, max_waves);
-  int chunk_per_wave = 1;
+  // Partials with rows on multiples of four elements (the library's own layout) are parked finished -- normalised,
+  // in mid_dtype, the rows of the real heads only: 2 KB for 8 heads in bf16 against 8.3 KB of raw state -- and a
+  // wave walks up to four splits; else the raw state is parked and normalised when it is stored.
+  const int hb_slots = a.hbsz > 16 ? 32 : 16;
+  const bool park_final = a.vec_out != 0;
+  // What a wish of `wish` consecutive splits per work item becomes: the waves of a head take whole splits,
+  // kMaxSplitsPerWave at most -- a wave keeps the finished partials of all but its last split in LDS until it has
+  // issued its last load (stores and loads of a wave retire in order, so a store between two tiles would hold back
+  // the loads behind it) --, so the chunk is a multiple of the waves, rounded down or up.  wgs: (sequence, work item,
+  // KV head, head block) units before that rounding, which the choices that follow were tuned with; grid_waves: the
+  // waves the grid will hold.
+  struct ChunkPlan { int chunk, waves, per_wave; int64_t wgs, grid_waves; };
+  auto chunk_plan = [&](int wish, bool round_up) {
+    ChunkPlan c;
+    const int items = (a.S + wish - 1) / wish;   // work items per (sequence, KV head, head block)
+    // Ranges that are certain to be busy per sequence: all of them, or, when the ranges follow each sequence's own
+    // length, only the ones every sequence gets (the rest of the grid may be empty ranges).
+    const int busy_splits = a.adapt > 0 && a.adapt < a.S ? a.adapt : items;
+    c.wgs = (int64_t)batch * busy_splits * a.Hkv * a.nhb;
+    c.waves = p->waves_per_block ? (p->waves_per_block < max_waves ? p->waves_per_block : max_waves)
+                                 : choose_waves(c.wgs, max_tok_split * wish, tile, wave_target, max_waves);
+    c.per_wave = 1;
+    c.chunk = wish;
+    if (wish > 1) {
+      while (c.waves > 1 && c.waves > wish) c.waves >>= 1;
+      c.per_wave = round_up ? (wish + c.waves - 1) / c.waves : wish / c.waves;
+      const int cap = park_final ? kMaxSplitsPerWaveFinal : kMaxSplitsPerWave;
+      if (c.per_wave > cap) c.per_wave = cap;
+      c.chunk = c.waves * c.per_wave;
+    }
+    c.grid_waves = (int64_t)batch * ((a.S + c.chunk - 1) / c.chunk) * a.Hkv * a.nhb * c.waves;
+    return c;
+  };
+  // Chunked work items: the caller's split count and ranges are kept exactly (they are observable in out_split), but a
+  // workgroup walks `chunk` consecutive splits, so that the chip sees about as many work items as the library's own
+  // plan would launch: every work item pays the prologue (arguments -> length -> block table -> first rows) once, not
+  // once per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.
+  // Not for large batches: their lengths differ in practice, and many short work items balance better over the CUs
+  // than few long ones (config 4's ragged batch of 64 with exactly 32 splits: 691 us unchunked, 713 us chunked).
+  ChunkPlan cp = chunk_plan(1, false);
+  if (use_mfma && D == 128 && Dv == D && !fuse && a.adapt == 0 && !a.order_items && !skip_empty && !no_lse && a.S > 1 &&
+      batch <= kMaxChunkBatch && !env_no_chunk()) {
+    fd_params plan = *p;
+    plan.split_adapt = 0;
+    const int s_plan = fd_plan_splits(&plan, batch);
+    if (s_plan > 0 && s_plan < a.S) {
+      // Splits per work item: the split count over the plan's, rounded up -- few long work items -- unless that
+      // leaves the grid short of the waves that keep the memory system busy (a split count the plan does not divide:
+      // 12 splits against a plan of 8 as 6 items of two are 768 waves on config 2's shape, 55 us; as 12 items 48 us;
+      // one sequence of 131072 tokens with 24 splits 148 against 95 us), then rounded down: at least as many items as
+      // the plan has.
+      cp = chunk_plan((a.S + s_plan - 1) / s_plan, true);
+      if (cp.grid_waves < wave_target * 7 / 8) cp = chunk_plan(a.S / s_plan, false);
+    }
+  }
+  a.chunk = cp.chunk;
+  max_tok_split *= a.chunk;
+  const int64_t wgs = cp.wgs;
+  int waves = cp.waves;
+  int chunk_per_wave = cp.per_wave;
   if (a.chunk > 1) {
-    // The waves of a head take whole splits, kMaxSplitsPerWave at most: a wave keeps the finished partials of all but
-    // its last split in LDS until it has issued its last load (stores and loads of a wave retire in order, so a store
-    // between two tiles would hold back the loads behind it).
-    while (waves > 1 && waves > a.chunk) waves >>= 1;
-    // Partials with rows on multiples of four elements (the library's own layout) are parked finished -- normalised,
-    // in mid_dtype, the rows of the real heads only: 2 KB for 8 heads in bf16 against 8.3 KB of raw state -- and a
-    // wave walks up to four splits; else the raw state is parked and normalised when it is stored.
-    const int hb_slots = a.hbsz > 16 ? 32 : 16;
-    a.park_final = a.vec_out;
+    a.park_final = park_final;
     a.park_bytes = a.park_final ? hb_slots * 4 + a.hbsz * D * msz : (hb_slots * D + 2 * hb_slots) * 4;
-    chunk_per_wave = (a.chunk + waves - 1) / waves;
-    const int cap = a.park_final ? kMaxSplitsPerWaveFinal : kMaxSplitsPerWave;
-    if (chunk_per_wave > cap) chunk_per_wave = cap;
-    a.chunk = waves * chunk_per_wave;
     a.park = chunk_per_wave - 1;
   }
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).
