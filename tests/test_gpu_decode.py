@@ -769,7 +769,8 @@ def test_fp8_d256_dequant_table_and_soft_cap(fd):
 # ---- scheduler
 def test_schedule_orders_longest_first(fd):
     gen = torch.Generator(device="cpu").manual_seed(71)
-    for B in (1, 2, 3, 64, 300, 1025, 2047, 2049, 5000):   # 2048 lengths go through LDS at a time
+    # (2048 lengths go through LDS at a time; 64 lanes share a sequence up to 2048 of them, fewer beyond)
+    for B in (1, 2, 3, 64, 300, 1025, 2047, 2048, 2049, 5000, 20000, 65535):
         lens = torch.randint(-3 if B == 300 else 0, 50, (B,), generator=gen, dtype=torch.int32)
         order = fd.schedule_sequences(lens.to(DEV)).cpu()
         expect = torch.argsort(lens, descending=True, stable=True).to(torch.int32)
