@@ -278,42 +278,15 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
   }
 }
 
-// order[rank] = sequence index, sequences ranked by kv_len descending, ties by index.  A sequence's rank is the number
-// of sequences in front of it.  T = 1 << t_shift lanes of a wave share a sequence (T is the same for the whole grid):
-// the lengths go through LDS in chunks, lane `part` of a sequence compares it with the groups of four lengths part,
-// part + T, ... of every chunk (lanes of one sequence read consecutive 16-byte groups, lanes of different sequences the
-// same ones), and the partial ranks are summed over the T lanes with shuffles.  With one thread per sequence walking all
-// the others 1024 sequences took 51 us -- one wave per SIMD on four CUs, every compare a dependent step.
-constexpr int kRankChunk = 2048;
-
+// order[rank] = sequence index, sequences ranked by kv_len descending, ties by index (fd_rank_sequence).
 __global__ void __launch_bounds__(256) fd_schedule_kernel(const int32_t* __restrict__ kv_lens, int batch, int t_shift,
                                                           int32_t* __restrict__ order) {
   __shared__ __align__(16) int32_t s_len[kRankChunk];
-  const int T = 1 << t_shift;
   const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  int mine;
+  const int rank = fd_rank_sequence(gid, batch, t_shift, [&](int j) { return kv_lens[j]; }, s_len, &mine);
   const int i = gid >> t_shift;
-  const int part = gid & (T - 1);
-  const int mine = i < batch ? kv_lens[i] : 0;
-  int rank = 0;
-  for (int j0 = 0; j0 < batch; j0 += kRankChunk) {
-    const int cnt = min(kRankChunk, batch - j0);
-    const int groups = (cnt + 3) >> 2;
-    __syncthreads();
-    // padding entries (INT32_MIN at indices >= batch) never rank before a real sequence
-    for (int j = threadIdx.x; j < 4 * groups; j += blockDim.x) s_len[j] = j < cnt ? kv_lens[j0 + j] : INT32_MIN;
-    __syncthreads();
-    for (int g = part; g < groups; g += T) {
-      const i32x4 other = *(const i32x4*)&s_len[4 * g];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) rank += (other[e] > mine) || (other[e] == mine && j0 + 4 * g + e < i);
-    }
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const int up = __shfl_xor(rank, off);
-    if (off < T) rank += up;
-  }
-  if (part == 0 && i < batch) order[rank] = i;
+  if ((gid & ((1 << t_shift) - 1)) == 0 && i < batch) order[rank] = i;
 }
 
 // One workgroup: the (sequence, range) issue order of a decode step (fd_schedule_items_block).
@@ -369,9 +342,7 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
 }
 
 int fd_launch_schedule(hipStream_t stream, const int32_t* kv_lens, int batch, int32_t* order) {
-  // lanes per sequence: as many as keep the grid at 512 workgroups or fewer (64 up to 2048 sequences, 2 at 65535)
-  int t_shift = 6;
-  while (t_shift > 0 && ((int64_t)batch << t_shift) > 131072) --t_shift;
+  const int t_shift = fd_rank_shift(batch);
   const unsigned grid = (unsigned)((((int64_t)batch << t_shift) + 255) / 256);
   hipLaunchKernelGGL(fd_schedule_kernel, dim3(grid), dim3(256), 0, stream, kv_lens, batch, t_shift, order);
   return hipGetLastError() == hipSuccess ? FD_OK : FD_ERR_LAUNCH;

@@ -128,6 +128,7 @@ struct AppendArgs {
   int32_t* items;        // nullptr or [2 * batch * ranges.S]: work items of the decode that follows (fd_schedule_items)
   RangePlan ranges;      // how that decode cuts a sequence into ranges (items only)
   int32_t data_blocks;   // workgroups that move data; the ones after them compute seq_order
+  int32_t rank_shift;    // log2 of the lanes that share a sequence in those (fd_rank_shift)
   const float* k_scale;
   const float* v_scale;
   int64_t skn_b, skn_t, skn_h, svn_b, svn_t, svn_h, sk_t, sk_h, sv_t, sv_h, sbt;
@@ -1062,6 +1063,54 @@ __device__ __forceinline__ void fused_combine(const SplitArgs& a, const WorkItem
       if (a.flse) a.flse[(int64_t)w.b * a.Hq + head] = lse;
     }
   }
+}
+
+// Rank of a sequence = the number of sequences in front of it when they are sorted by length descending, ties by
+// index.  T = 1 << t_shift lanes of a wave share a sequence (T is the same for the whole ranking grid, whose thread
+// `gid` serves sequence gid >> t_shift): the lengths go through LDS in chunks, lane `part` of a sequence compares it with
+// the groups of four lengths part, part + T, ... of every chunk (lanes of one sequence read consecutive 16-byte groups,
+// lanes of different sequences the same ones), and the partial ranks are summed over the T lanes with shuffles.  With
+// one thread per sequence walking all the others 1024 sequences took 51 us -- one wave per SIMD on four CUs, every
+// compare a dependent step.  Every thread of the workgroup calls this (it contains barriers); the result is valid in
+// all T lanes of sequences < batch.  s_len: LDS, kRankChunk entries, 16-byte aligned.  len_of(j): length of sequence j.
+constexpr int kRankChunk = 2048;
+
+template <typename LenFn>
+__device__ __forceinline__ int fd_rank_sequence(int gid, int batch, int t_shift, LenFn len_of, int32_t* s_len,
+                                                int* mine_out) {
+  const int T = 1 << t_shift;
+  const int i = gid >> t_shift;
+  const int part = gid & (T - 1);
+  const int mine = i < batch ? len_of(i) : 0;
+  int rank = 0;
+  for (int j0 = 0; j0 < batch; j0 += kRankChunk) {
+    const int cnt = min(kRankChunk, batch - j0);
+    const int groups = (cnt + 3) >> 2;
+    __syncthreads();
+    // padding entries (INT32_MIN at indices >= batch) never rank before a real sequence
+    for (int j = threadIdx.x; j < 4 * groups; j += blockDim.x) s_len[j] = j < cnt ? len_of(j0 + j) : INT32_MIN;
+    __syncthreads();
+    for (int g = part; g < groups; g += T) {
+      const i32x4 other = *(const i32x4*)&s_len[4 * g];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rank += (other[e] > mine) || (other[e] == mine && j0 + 4 * g + e < i);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const int up = __shfl_xor(rank, off);
+    if (off < T) rank += up;
+  }
+  *mine_out = mine;
+  return rank;
+}
+
+// Lanes per sequence for fd_rank_sequence: as many as keep the ranking grid at 512 workgroups of 256 threads or fewer
+// (64 up to 2048 sequences, 2 at 65535).
+inline int fd_rank_shift(int64_t batch) {
+  int t_shift = 6;
+  while (t_shift > 0 && (batch << t_shift) > 131072) --t_shift;
+  return t_shift;
 }
 
 // Sequences one scheduling workgroup ranks (its LDS holds 12 bytes per sequence).

@@ -139,16 +139,15 @@ __global__ __launch_bounds__(256) void fd_kv_append_kernel(const AppendArgs a) {
       return;
     }
     // per-sequence order: grown length descending, ties by index
-    const int i = ((int)blockIdx.x - a.data_blocks) * blockDim.x + threadIdx.x;
-    if (i >= a.batch) return;
-    const int64_t mine = grown(i);
-    int rank = 0;
-    for (int j = 0; j < a.batch; ++j) {
-      const int64_t other = grown(j);
-      rank += (other > mine) || (other == mine && j < i);
+    __shared__ __align__(16) int32_t s_len[kRankChunk];
+    const int gid = ((int)blockIdx.x - a.data_blocks) * blockDim.x + threadIdx.x;
+    int mine;
+    const int rank = fd_rank_sequence(gid, a.batch, a.rank_shift, [&](int b) { return (int)grown(b); }, s_len, &mine);
+    const int i = gid >> a.rank_shift;
+    if ((gid & ((1 << a.rank_shift) - 1)) == 0 && i < a.batch) {
+      a.seq_order[rank] = i;
+      a.seq_order[a.batch + rank] = mine;   // the lengths in issue order, for the decode's prologue
     }
-    a.seq_order[rank] = i;
-    a.seq_order[a.batch + rank] = (int32_t)mine;   // the lengths in issue order, for the decode's prologue
     return;
   }
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -246,7 +245,8 @@ int fd_launch_kv_append(hipStream_t stream, const AppendArgs& args, int src_dtyp
     if (a.batch > 256) return FD_ERR_TOO_LARGE;
     blocks += 1;
   } else if (a.seq_order) {
-    blocks += (a.batch + 255) / 256;
+    a.rank_shift = fd_rank_shift(a.batch);
+    blocks += (((int64_t)a.batch << a.rank_shift) + 255) / 256;
   }
   const dim3 grid((unsigned)blocks);
   switch (src_dtype) {

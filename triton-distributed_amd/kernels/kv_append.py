@@ -162,8 +162,8 @@ def apply_rotary_pos_emb(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: t
 
 _ARANGE = {}
 # Batches for which flash_attn_with_kvcache lets the append launch rank the sequences: below, every sequence's
-# workgroups start at once anyway; above, one thread per sequence ranking against all others gets long.
-SCHEDULE_MIN_BATCH, SCHEDULE_MAX_BATCH = 16, 1024
+# workgroups start at once anyway; the upper end is what ``seq_order_out`` takes.
+SCHEDULE_MIN_BATCH, SCHEDULE_MAX_BATCH = 16, 4096
 
 
 def _dense_block_table(device, n):
