@@ -413,7 +413,7 @@ def main():
     lse_split = split_ws[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
     hstream = torch.cuda.current_stream().cuda_stream
     order_ptr = None
-    if args.variant == "persistent" and not args.exact_splits and S_eff > 1 and p.split_adapt > 0 and B <= fk.MAX_ITEM_BATCH:
+    if args.variant == "persistent" and not args.exact_splits and S_eff > 1 and p.split_adapt > 0 and B <= fk.ITEMS_UP_TO_BATCH:
         # the issue order the scheduled step uses: (sequence, range) items, computed once for this leg
         items = fk.item_order_buffer(B, S_eff, dev)
         fd._lib.check(lib.fd_schedule_items(hstream, wl.kv_lens.data_ptr(), B, items.data_ptr(), byref(p)))

@@ -20,7 +20,7 @@ from typing import Optional, Tuple, Union
 import torch
 
 from .._lib import FdParams, FdQkPrep, check, fd_dtype_of, load_library, stream_handle
-from .flash_decode import (MAX_FUSED_ITEM_BATCH, SPLIT_ALIGN, _decode, _require_cuda, item_order_buffer,
+from .flash_decode import (ITEMS_UP_TO_BATCH, SPLIT_ALIGN, _decode, _require_cuda, item_order_buffer,
                            plan_decode)
 
 
@@ -237,7 +237,7 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
                                    k_scale=k_scale, v_scale=v_scale, path=decode_kw.get("path", "auto"),
                                    waves_per_block=decode_kw.get("waves_per_block", 0),
                                    max_kv_len=decode_kw.get("max_kv_len"))
-            if S > 1 and adapt > 0 and bsz <= MAX_FUSED_ITEM_BATCH and not decode_kw.get("fuse_combine"):
+            if S > 1 and adapt > 0 and bsz <= ITEMS_UP_TO_BATCH and not decode_kw.get("fuse_combine"):
                 items, item_plan = item_order_buffer(bsz, S, dev), (S, SPLIT_ALIGN, adapt)
                 decode_kw["item_order"] = items
             else:
