@@ -1010,13 +1010,14 @@ def test_large_batch_single_split_direct_output(fd, kind, variant):
         assert_out_close(res[..., :D].cpu(), ref, atol=atol)
         # the LSE column has the output's dtype
         assert_lse_close(res[..., D].float().cpu(), ref_lse, rtol=1e-5 if dtype == torch.float32 else 1e-2)
-    # two launches on the same inputs (exactly one split into a caller buffer, then the combine): same bits
+    # two launches on the same inputs (exactly one split into a caller buffer, then the combine): same bits, given
+    # the same waves per range (the planner's own choice differs between a planned and a literal split count)
     if not fp8:
         two = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
                                       kv_split=1, output_split=torch.empty(B, Hq, 1, D + 1, dtype=torch.float32,
-                                                                           device=DEV))
+                                                                           device=DEV), waves_per_block=1)
         one = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale,
-                                      kv_split=32)
+                                      kv_split=32, waves_per_block=1)
         torch.cuda.synchronize()
         assert torch.equal(one.cpu().view(torch.uint8), two.cpu().view(torch.uint8))
 
