@@ -15,7 +15,8 @@ Keyword-only additions that the reference does not have (all default off):
   extra_partials  (out [E,B,Hq,Dv], lse [E,B,Hq] fp32): further partials merged by
                   the combine, standing in for what other sequence-parallel ranks
                   would contribute
-  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences
+  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (batches of
+                  ``AUTO_ORDER_FROM_BATCH`` = 128 sequences or more are ranked by the wrapper itself when none is given)
   seq_order_lens  int32 [B], with ``seq_order``: ``kv_lens[seq_order]`` (``rope_kv_append`` writes both), which
                   saves a workgroup one dependent load before it can start
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
@@ -186,6 +187,10 @@ MAX_SEQ_ORDER_BATCH = 4096  # sequences the scheduled variant ranks with fd_sche
 # more than it gains over the per-sequence order (256 ragged sequences of up to 8192 tokens: 650 against 640 us,
 # 160 of them: 426 against 435 us)
 ITEMS_UP_TO_BATCH = 192
+# From this batch size on the plain wrappers rank the sequences as well (one launch of 3.5 us): a batch that large is
+# ragged in practice and runs 8 - 15 % faster longest first (256 sequences of up to 2048 tokens: 187 against 159 us),
+# a uniform one loses the launch.  0 switches it off; callers that pass ``seq_order`` / ``item_order`` are not touched.
+AUTO_ORDER_FROM_BATCH = 128
 
 
 def _hint(max_kv_len, capacity):
@@ -306,7 +311,9 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
     want_items = (item_order is not None or schedule_items) and num_splits > 1 and not fuse_combine
     if want_items and item_order is None and batch > ITEMS_UP_TO_BATCH:
         want_items = False
-    if schedule_items and not want_items and seq_order is None and 1 < batch <= MAX_SEQ_ORDER_BATCH:
+    auto_order = (AUTO_ORDER_FROM_BATCH and batch >= AUTO_ORDER_FROM_BATCH and not no_alloc
+                  and block_table.shape[1] * page_size >= 1024)
+    if (schedule_items or auto_order) and not want_items and seq_order is None and 1 < batch <= MAX_SEQ_ORDER_BATCH:
         # per-sequence order where items do not apply -- a single split per sequence (256 ragged sequences of up to
         # 2048 tokens: 187 us in index order, 156 us longest first), the fused combine, batches beyond the item
         # scheduler's; still larger batches are left to the dispatcher
