@@ -373,12 +373,12 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     // other MFMA kernels alike, scheduled: head_dim 64 40 sequences of up to 16384 tokens 134 -> 116 us, fp8 head_dim
     // 256 96 of up to 8192 tokens 321 -> 280 us, fp8 head_dim 128 256 of up to 2048 tokens in one split 98 -> 87 us;
     // not the fp8 head_dim-64 kernel, whose waves serve two KV heads each).
-    // Four in a small batch whose full-length ranges have 3072 tokens or more (16-bit caches): its few longest
-    // sequences are the last to finish, and their waves alone must keep the memory busy (16 ragged sequences of up to
-    // 32768 tokens 166 -> 149 us; from 32 sequences on it gains nothing, and config 5's fp8 step lost 6 % to it: four
-    // waves per range leave room for two sibling KV heads instead of four).
+    // Four in a small batch whose full-length ranges have 3072 tokens or more: its few longest sequences are the last
+    // to finish, and their waves alone must keep the memory busy (16 ragged sequences of up to 32768 tokens 166 -> 149
+    // us, on an fp8 cache with 64 query heads 108 -> 88 us; from 32 sequences on it gains nothing, and config 5's fp8
+    // step lost 6 % to it: four waves per range leave room for two sibling KV heads instead of four).
     if (use_mfma && !(kv_fp8 && D == 64) && a.adapt > 0 && batch > 1 && !p->waves_per_block && env_waves() == 0) {
-      const int at_least = D == 128 && a.S > 1 && !kv_fp8 && batch <= 24 && max_tok_split * wish >= kMaxTokensPerRange * 3 / 4 && max_waves >= 4 ? 4 : 2;
+      const int at_least = D == 128 && a.S > 1 && batch <= 24 && max_tok_split * wish >= kMaxTokensPerRange * 3 / 4 && max_waves >= 4 ? 4 : 2;
       if (c.waves < at_least && max_tok_split * wish >= at_least * tile) c.waves = at_least;
     }
     c.per_wave = 1;
