@@ -318,6 +318,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         # 2048 tokens: 187 us in index order, 156 us longest first), the fused combine, batches beyond the item
         # scheduler's; still larger batches are left to the dispatcher
         seq_order = schedule_sequences(kv_lens, stream=stream)
+        if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
+            seq_order.record_stream(stream)
     # internal partials: splits may start on tile boundaries (the ranges are not observable)
     p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
                      v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
