@@ -416,7 +416,6 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     }
   }
   a.chunk = cp.chunk;
-  max_tok_split *= a.chunk;
   const int64_t wgs = cp.wgs;
   int waves = cp.waves;
   int chunk_per_wave = cp.per_wave;
