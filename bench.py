@@ -174,7 +174,7 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     """Every north-star figure besides the headline, in this same process, each as (microseconds per decode step,
     fraction of the 8 TB/s peak on the step's algorithmic bytes): config 2 with exactly the 32 splits the workload
     names; config 5 (fp8 KV) and its bf16 twin, planned and with exactly 64 splits, and their ratios (target >= 1.7);
-    config 3, planned and with exactly 32 splits; config 4 scheduled and unscheduled."""
+    config 3, planned and with exactly 32 splits; config 4 scheduled, through the plain wrapper and unscheduled."""
     U = fd.utils
     t = {}
     # the headline times exactly the steps the command line asks for; these side figures take at least 100 steps and
@@ -203,7 +203,15 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     c4 = U.make_config(4)
     n4 = steps // 4   # a step of config 4 is 15 times config 2's
     put("c4_ragged_scheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0, variant="persistent"))
-    put("c4_ragged_unscheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
+    # the plain wrapper ranks the sequences of a batch this large itself; "unscheduled" is that wrapper with the
+    # ranking switched off: sequences issued in index order
+    put("c4_ragged_plain_wrapper", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
+    fk = _flash_decode(fd)
+    auto_order, fk.AUTO_ORDER_FROM_BATCH = fk.AUTO_ORDER_FROM_BATCH, 0
+    try:
+        put("c4_ragged_unscheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
+    finally:
+        fk.AUTO_ORDER_FROM_BATCH = auto_order
     del c4
     return t
 

@@ -16,7 +16,7 @@ Keyword-only additions that the reference does not have (all default off):
                   the combine, standing in for what other sequence-parallel ranks
                   would contribute
   seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (batches of
-                  ``AUTO_ORDER_FROM_BATCH`` = 128 sequences or more are ranked by the wrapper itself when none is given)
+                  ``AUTO_ORDER_FROM_BATCH`` = 64 sequences or more are ranked by the wrapper itself when none is given)
   seq_order_lens  int32 [B], with ``seq_order``: ``kv_lens[seq_order]`` (``rope_kv_append`` writes both), which
                   saves a workgroup one dependent load before it can start
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
@@ -188,9 +188,10 @@ MAX_SEQ_ORDER_BATCH = 4096  # sequences the scheduled variant ranks with fd_sche
 # 160 of them: 426 against 435 us)
 ITEMS_UP_TO_BATCH = 192
 # From this batch size on the plain wrappers rank the sequences as well (one launch of 3.5 us): a batch that large is
-# ragged in practice and runs 8 - 15 % faster longest first (256 sequences of up to 2048 tokens: 187 against 159 us),
-# a uniform one loses the launch.  0 switches it off; callers that pass ``seq_order`` / ``item_order`` are not touched.
-AUTO_ORDER_FROM_BATCH = 128
+# ragged in practice and runs 4 - 15 % faster longest first (256 sequences of up to 2048 tokens: 187 against 159 us,
+# 72 of up to 8192 tokens 213 against 196 us), a uniform one loses the launch.  0 switches it off; callers that pass
+# ``seq_order`` / ``item_order`` are not touched.
+AUTO_ORDER_FROM_BATCH = 64
 
 
 def _hint(max_kv_len, capacity):
