@@ -103,8 +103,11 @@ def _flash_decode(fd):
     return importlib.import_module(fd.__name__ + ".kernels.flash_decode")
 
 
-def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="auto", waves=0, fuse=False):
-    """The decode step of a workload as a callable of the step index, plus its output and LSE tensors."""
+def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="auto", waves=0, fuse=False,
+              caller_partials=None):
+    """The decode step of a workload as a callable of the step index, plus its output and LSE tensors.
+    caller_partials: a dtype -- the caller hands in ``output_split [B, Hq, S, D + 1]`` of that type, as the reference's
+    sequence-parallel layer does on every call (sp_flash_decode_layer.py:95-110): exactly S observable partials."""
     B, Hq, D = wl.q.shape
     out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
@@ -120,6 +123,8 @@ def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="
         kw.update(extra_partials=(wl.extra_out, wl.extra_lse))
     if exact:
         kw["plan_splits"] = False
+    if caller_partials is not None:
+        kw["output_split"] = torch.empty(B, Hq, S, D + 1, dtype=caller_partials, device=dev)
     fn = fd.gqa_fwd_batch_decode_persistent if variant == "persistent" else fd.gqa_fwd_batch_decode
 
     def step(i):   # persistent: the scheduling launch is part of the step (inside the wrapper)
@@ -153,7 +158,8 @@ def settle(torch, step, ramp_ms):
     return (time.perf_counter() - t_ramp) * 1e3
 
 
-def measure_target(torch, fd, dev, wl_cpu, steps, warmup, pools_n, ramp_ms, resident=None, **step_kw):
+def measure_target(torch, fd, dev, wl_cpu, steps, warmup, pools_n, ramp_ms, resident=None, step_factory=None,
+                   **step_kw):
     """One north-star target measured the way the headline is: the whole decode step (split + combine) of a
     workload, rotating over independent pools, after the clocks have settled.  Its pools go back to torch's
     caching allocator, not to the driver: a GPU that has just been handed back gigabytes is slow for a few seconds
@@ -163,11 +169,61 @@ def measure_target(torch, fd, dev, wl_cpu, steps, warmup, pools_n, ramp_ms, resi
     else:
         wl = wl_cpu.to(dev)
         pools = make_pools(torch, wl, dev, pools_n)
-    step, _, _, _ = make_step(torch, fd, wl, pools, wl.kv_split, dev, **step_kw)
+    if step_factory is not None:   # another caller of the path: step_factory(workload, pools) -> step(i)
+        step = step_factory(wl, pools)
+    else:
+        step, _, _, _ = make_step(torch, fd, wl, pools, wl.kv_split, dev, **step_kw)
     settle(torch, step, ramp_ms)
     us = _time_us(torch, step, steps, warmup)
     nbytes = wl_cpu.algorithmic_bytes()
     return round(us, 3), round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+
+
+def _binding_step(torch, fd, dev):
+    """The decode step through ``reference_binding.gqa_fwd_batch_decode`` (positional reference signature)."""
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.abspath(fd.__file__)), "reference_binding.py")
+    spec = importlib.util.spec_from_file_location("fd_reference_binding_bench", path)
+    rb = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(rb)
+
+    def factory(wl, pools):
+        B, Hq, D = wl.q.shape
+        S = wl.kv_split
+        out_split = torch.empty(B, Hq, S, D + 1, dtype=torch.float32, device=dev)
+        out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
+        q_lens = [1] * B
+
+        def step(i):
+            k, v = pools[i % len(pools)]
+            return rb.gqa_fwd_batch_decode(wl.q, k, v, None, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap,
+                                           out_split, out, S)
+        return step
+    return factory
+
+
+def _sp_layer_step(torch, fd, dev, reference_settings):
+    """``SpGQAFlashDecodeAttention(num_ranks=8).forward`` on one rank's shard with the other ranks' partials given."""
+    def factory(wl, pools):
+        B, Hq, D = wl.q.shape
+        _, P, Hkv, _ = wl.k_cache.shape
+        R = wl.extra_out.shape[0] + 1
+        layer = fd.SpGQAFlashDecodeAttention(0, 0, R, 1, Hq, Hkv, D, D, page_size=P, scale=wl.scale,
+                                             soft_cap=wl.soft_cap, max_allowed_batch=B,
+                                             **({"partial_dtype": None} if reference_settings else {}))
+        out_split = None
+        if reference_settings:
+            layer.kv_split = 32                                    # sp_flash_decode_layer.py:62
+            out_split = torch.empty(B, Hq, 32, D + 1, dtype=wl.q.dtype, device=dev)   # :95-96
+        lens = torch.ones(R, B, dtype=torch.int32, device=dev)
+        lens[0] = wl.kv_lens
+        remote = (wl.extra_out, wl.extra_lse)
+
+        def step(i):
+            k, v = pools[i % len(pools)]
+            return layer(wl.q, k, v, lens, wl.block_table, remote_partials=remote, output_split=out_split)
+        return step
+    return factory
 
 
 def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
@@ -188,7 +244,19 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     # decides how far the address translation reaches, which is worth a few per cent at this size)
     put("c2_exact_32_splits", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
                                              resident=c2_resident, exact=True))
+    # the reference's literal call: the caller owns the partials, [B, Hq, 32, D + 1] (sp_flash_decode_layer.py:95-110
+    # allocates them in q.dtype; the perf scripts in fp32, test_decode_attn.py:322) -- exactly 32 observable partials
+    put("c2_caller_partials_fp32", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
+                                                  resident=c2_resident, caller_partials=torch.float32))
+    put("c2_caller_partials_bf16", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
+                                                  resident=c2_resident, caller_partials=torch.bfloat16))
+    # ... and through the stand-alone ctypes binding a maintainer of the reference tree would add (fp32 partials of
+    # its own, no plan, nothing of this package's Python between the call and the library)
+    put("c2_reference_binding", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
+                                               resident=c2_resident, step_factory=_binding_step(torch, fd, dev)))
     c5, c5t = U.make_config(5), U.make_config5_bf16_twin()
+    put("c5_caller_partials_bf16", measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0,
+                                                  caller_partials=torch.bfloat16))
     put("c5_fp8", measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0))
     put("c5_fp8_exact_64_splits", measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0, exact=True))
     put("c5_bf16_twin", measure_target(torch, fd, dev, c5t, steps, warmup, 4, 100.0))
@@ -199,6 +267,13 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     c3 = U.make_config(3)
     put("c3_sp_shard_plus_7_partials", measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0))
     put("c3_exact_32_splits", measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0, exact=True))
+    # the caller of the path: SpGQAFlashDecodeAttention.forward on this shard as rank 0 of 8, the 7 seeded partials
+    # standing in for what the other ranks' allgather would deliver -- with the layer's defaults, and with the
+    # reference's settings (32 splits, partials visible to the caller and staged in q.dtype)
+    put("c3_sp_layer_forward", measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0,
+                                              step_factory=_sp_layer_step(torch, fd, dev, False)))
+    put("c3_sp_layer_forward_reference_settings",
+        measure_target(torch, fd, dev, c3, steps, warmup, 4, 100.0, step_factory=_sp_layer_step(torch, fd, dev, True)))
     del c3
     c4 = U.make_config(4)
     n4 = steps // 4   # a step of config 4 is 15 times config 2's
@@ -376,6 +451,7 @@ def main():
     for i in range(args.steps):
         step(i)
     e1.record()
+    issue_us = (time.perf_counter() - t0) * 1e6 / (args.steps + 1)   # host time to enqueue a step (nothing waited for)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 * args.steps / (args.steps + 1)   # host clock over steps + 1 calls
     gpu_ms = e0.elapsed_time(e1)
@@ -503,6 +579,9 @@ def main():
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
+        # the host's own share: wall time per step up to the last enqueue, before the synchronize (the wall figure
+        # above ends after it and so can never be below the GPU's time per step)
+        "host_issue_us_per_step": round(issue_us, 3),
         "hip_graph_replay_us_per_step": None if graph_us is None else round(graph_us, 3),
         "clock_ramp_ms": round(ramp_ms),
         "timing": "HIP events around exactly `steps` back-to-back steps; 1 untimed lead-in step between the "
