@@ -104,19 +104,24 @@ def _flash_decode(fd):
 
 
 def make_step(torch, fd, wl, pools, S, dev, variant="plain", exact=False, path="auto", waves=0, fuse=False,
-              caller_partials=None):
+              caller_partials=None, auto_order=True):
     """The decode step of a workload as a callable of the step index, plus its output and LSE tensors.
     caller_partials: a dtype -- the caller hands in ``output_split [B, Hq, S, D + 1]`` of that type, as the reference's
     sequence-parallel layer does on every call (sp_flash_decode_layer.py:95-110): exactly S observable partials."""
     B, Hq, D = wl.q.shape
     out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
-    # kv_split -1: the library chooses the split count and owns the partials
-    # room for the partials of as many splits as the step may be planned with
-    S_ws = max(S, 0) if exact else _flash_decode(fd).split_bound(S, wl.block_table.shape[1] * wl.k_cache.shape[1])
-    workspace = torch.empty(B * Hq * S_ws * (D + 1), dtype=torch.float32, device=dev) if S_ws > 0 else None
+    # the workspace the library asks for (partials, their LSEs, the issue order): with it the step allocates nothing
+    fk, L = _flash_decode(fd), fd._lib
+    flags = (L.FD_STEP_EXACT_SPLITS if exact else 0) | (L.FD_STEP_SCHEDULE if variant == "persistent" else 0) \
+        | (0 if auto_order else L.FD_STEP_NO_ORDER) | (L.FD_STEP_FUSED if fuse else 0)
+    need = fk.workspace_bytes(wl.q, wl.k_cache, wl.block_table, S, flags=flags, fp8=wl.k_scale is not None, path=path,
+                              waves_per_block=waves, num_extra=0 if wl.extra_out is None else wl.extra_out.shape[0])
+    workspace = torch.empty(max(need, 4) // 4 + 64, dtype=torch.float32, device=dev)
     q_lens = [1] * B
     kw = dict(output_combine=out, kv_split=S, lse_out=lse, path=path, waves_per_block=waves, fuse_combine=fuse)
+    if not auto_order:
+        kw["auto_order"] = False
     if wl.k_scale is not None:
         kw.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
     if wl.extra_out is not None:
@@ -281,12 +286,7 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     # the plain wrapper ranks the sequences of a batch this large itself; "unscheduled" is that wrapper with the
     # ranking switched off: sequences issued in index order
     put("c4_ragged_plain_wrapper", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
-    fk = _flash_decode(fd)
-    auto_order, fk.AUTO_ORDER_FROM_BATCH = fk.AUTO_ORDER_FROM_BATCH, 0
-    try:
-        put("c4_ragged_unscheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
-    finally:
-        fk.AUTO_ORDER_FROM_BATCH = auto_order
+    put("c4_ragged_unscheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0, auto_order=False))
     del c4
     return t
 
@@ -479,32 +479,31 @@ def main():
     from ctypes import byref
     lib = fd.load_library()
     fk = importlib.import_module("triton-distributed_amd.kernels.flash_decode")
-    S_bound = S
-    if not args.exact_splits:   # the library's own bound, as in the wrapper (the caller's count is a hint there)
-        S_bound = fk.split_bound(S, wl.block_table.shape[1] * wl.k_cache.shape[1])
-    p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_bound, wl.soft_cap, fd._lib.FD_F32, fd._lib.fd_dtype_of(out),
-                        wl.k_scale, wl.v_scale, args.path, args.waves)
-    p.split_align = fk.SPLIT_ALIGN                                        # as the step above: internal partials
-    S_eff = S_bound if args.exact_splits else lib.fd_plan_splits(byref(p), B)   # what the step above used
-    p.mid_dtype = fk.internal_partial_dtype(out.dtype, not args.exact_splits, args.fuse, B * Hq * S_eff * D)
-    if not args.exact_splits:
-        p.split_adapt = lib.fd_plan_min_splits(byref(p), B)
-    p.num_splits = S_eff
+    L = fd._lib
+    # the plan the step above ran with (fd_plan_decode), so that this leg launches the same split kernel
+    flags = (L.FD_STEP_EXACT_SPLITS if args.exact_splits else 0) | (L.FD_STEP_SCHEDULE if args.variant == "persistent" else 0) \
+        | (L.FD_STEP_FUSED if args.fuse else 0)
+    plan = fk.decode_plan(wl.q, wl.k_cache, wl.block_table, S, flags=flags, out_dtype=L.fd_dtype_of(out),
+                          fp8=wl.k_scale is not None, path=args.path, waves_per_block=args.waves,
+                          num_extra=0 if wl.extra_out is None else wl.extra_out.shape[0])
+    S_eff = plan.num_splits
+    p = fk._make_params(wl.q, wl.k_cache, wl.block_table, S_eff, wl.soft_cap, plan.mid_dtype, L.fd_dtype_of(out),
+                        wl.k_scale, wl.v_scale, args.path, args.waves, None, plan.split_align, plan.split_adapt)
     n_o = B * Hq * S_eff * D
-    split_ws = workspace if workspace is not None else torch.empty(B * Hq * S_eff * (D + 1), dtype=torch.float32,
-                                                                     device=dev)
+    split_ws = torch.empty(B * Hq * S_eff * (D + 1), dtype=torch.float32, device=dev)
     mid = split_ws[:n_o].view(B, Hq, S_eff, D)
     lse_split = split_ws[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
     hstream = torch.cuda.current_stream().cuda_stream
     order_ptr = None
-    if args.variant == "persistent" and not args.exact_splits and S_eff > 1 and p.split_adapt > 0 and B <= fk.ITEMS_UP_TO_BATCH:
+    if plan.order_kind == L.FD_ORDER_ITEMS:
         # the issue order the scheduled step uses: (sequence, range) items, computed once for this leg
         items = fk.item_order_buffer(B, S_eff, dev)
-        fd._lib.check(lib.fd_schedule_items(hstream, wl.kv_lens.data_ptr(), B, items.data_ptr(), byref(p)))
+        L.check(lib.fd_schedule_items(hstream, wl.kv_lens.data_ptr(), B, items.data_ptr(), byref(p)))
         p.seq_order_items = 1
         order_ptr = items.data_ptr()
-    elif args.variant == "persistent":
-        order_ptr = fd.schedule_sequences(wl.kv_lens).data_ptr()
+    elif plan.order_kind == L.FD_ORDER_SEQUENCES:
+        order_keep = fd.schedule_sequences(wl.kv_lens)
+        order_ptr = order_keep.data_ptr()
 
     def split_only(i):
         k, v = pools[i % len(pools)]
@@ -573,6 +572,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": wl.name, "batch": B, "q_heads": Hq, "kv_heads": wl.k_cache.shape[2], "head_dim": D,
                    "page_size": wl.k_cache.shape[1], "kv_splits": S, "kv_splits_used": S_eff,
+                   "launch_plan": dict(plan.launch, split_adapt=plan.split_adapt, split_align=plan.split_align,
+                                       partial_dtype=["f32", "f16", "bf16"][plan.mid_dtype],
+                                       order_kind=["none", "sequences", "items"][plan.order_kind],
+                                       workspace_bytes=plan.workspace_bytes),
                    "kv_len_total": int(wl_cpu.kv_lens.sum()), "kv_pools_rotated": len(pools),
                    "variant": args.variant, "path": args.path, "fused_combine": args.fuse},
         "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FD_ABI_VERSION 2
+#define FD_ABI_VERSION 3
 
 #if defined(__GNUC__)
 #define FD_API __attribute__((visibility("default")))
@@ -228,6 +228,121 @@ FD_API int fd_decode(void* stream, const void* q, const void* k_cache, const voi
               const int32_t* seq_order, int32_t combine_mode,
               const void* extra_out, const float* extra_lse, int32_t num_extra,
               int32_t* tickets, const fd_params* params);
+
+/*
+ * The launch policy of a decode step, in one place.  NUM_KV_SPLITS is a tuning constant in the reference (32 unless
+ * the caller says otherwise, flash_decode.py:779) and its wrappers allocate their partial buffers themselves
+ * (flash_decode.py:783-786); a caller that does not hand in `output_split` never sees the partials, so everything
+ * about them -- how many, which token ranges, their element type, where they live, in which order the work is issued
+ * -- is the library's choice.  fd_plan_decode reports that choice, fd_decode_planned applies it; a binding needs no
+ * policy of its own.
+ */
+typedef enum fd_step_flags {
+  FD_STEP_EXACT_SPLITS = 1,   /* exactly params->num_splits splits (the reference's ranges, rounded up to whole tiles)
+                                 instead of the library's count; the partials still live in the workspace           */
+  FD_STEP_SCHEDULE = 2,       /* the scheduled variant (gqa_fwd_batch_decode_persistent, flash_decode.py:931-1005):
+                                 the step ranks its work on the device first -- (sequence, range) work items up to
+                                 192 sequences, whole sequences up to 4096 -- and issues it largest first             */
+  FD_STEP_NO_ORDER = 4,       /* never rank: workgroups are issued in index order                                    */
+  FD_STEP_FUSED = 8,          /* fd_plan_decode only: plan for fd_decode with a ticket buffer (fp32 partials, no
+                                 work items, no direct single-split output)                                          */
+  FD_STEP_LSE_TWICE = 16,     /* fd_plan_decode only: the caller wants the merged LSE both in the output's column and
+                                 in lse_out, which the direct single-split output cannot provide                     */
+  FD_STEP_CALLER_PARTIALS = 32,/* fd_plan_decode only: the caller owns the partials ([B, Hq, S, Dv + 1] in
+                                 params->mid_dtype, flash_decode.py:783): exactly params->num_splits splits with the
+                                 reference's ranges; the plan only says how the step is issued                       */
+  FD_STEP_ORDER_FROM_APPEND = 64 /* fd_plan_decode only: an fd_kv_append launch precedes the step and can compute the
+                                 issue order in its trailing workgroups at no launch of its own; order_kind then
+                                 says which kind to ask it for (from 16 sequences on)                                */
+} fd_step_flags;
+
+typedef enum fd_order_kind {
+  FD_ORDER_NONE = 0,          /* index order                                                                        */
+  FD_ORDER_SEQUENCES = 1,     /* fd_schedule: [batch] sequence indices, longest first                               */
+  FD_ORDER_ITEMS = 2          /* fd_schedule_items: [2 * batch * num_splits] work items and their lengths           */
+} fd_order_kind;
+
+typedef struct fd_launch_plan {
+  int32_t num_splits;         /* grid slots (ranges) per sequence                                                   */
+  int32_t split_adapt;        /* fd_params.split_adapt of the step                                                  */
+  int32_t split_align;        /* fd_params.split_align of the step                                                  */
+  int32_t mid_dtype;          /* fd_dtype of the partials                                                           */
+  int32_t direct;             /* 1: one split and nothing else to merge -- the split kernel writes `out` itself, no
+                                 partials, no combine launch                                                        */
+  int32_t order_kind;         /* fd_order_kind of the scheduling launch the step makes itself (FD_ORDER_NONE when the
+                                 caller brings an order, asks for none, or the batch is not worth one)              */
+  int32_t mfma;               /* 1: an MFMA split kernel, 0: the VALU kernel                                        */
+  int32_t tile;               /* tokens per tile of that kernel                                                     */
+  int32_t waves_per_head;     /* waves that share the tokens of one (KV head or head block, work item)              */
+  int32_t members;            /* sibling KV heads (or head blocks, or V halves) per workgroup                       */
+  int32_t chunk;              /* consecutive splits one workgroup walks (1: a workgroup per split)                  */
+  int32_t head_block;         /* query-head slots a wave serves                                                     */
+  int32_t grid[3];            /* launch grid of the split kernel                                                    */
+  int32_t store_through;      /* 1: partials are written through to memory                                          */
+  int32_t max_kv_len;         /* the length hint the step is planned with (0: the block table's capacity)           */
+  int32_t reserved;
+  int64_t partial_bytes;      /* partials in the workspace ([batch, Hq, num_splits, Dv] in mid_dtype)               */
+  int64_t lse_bytes;          /* their fp32 LSEs ([batch, Hq, num_splits])                                          */
+  int64_t order_bytes;        /* the issue order                                                                    */
+  int64_t workspace_bytes;    /* all of it, each part on a 256-byte boundary                                        */
+} fd_launch_plan;
+
+/*
+ * The plan of a decode step for a shape known on the host (kv_lens is never read): split count and ranges, partial
+ * type, whether a scheduling launch is part of the step, the launch shape of the split kernel (for contiguous caches:
+ * token stride = kv_heads * head_dim, head stride = head_dim) and the workspace the step needs.  params->num_splits is
+ * the caller's hint -- <= 0: none; the reference's callers pass 32 -- which bounds the count from below only where it
+ * exceeds the library's own bound max(32, min(256, capacity / 512)); with FD_STEP_EXACT_SPLITS or
+ * FD_STEP_CALLER_PARTIALS it is the count (<= 0: 32).  params->mid_dtype, split_align, split_adapt and seq_order_items are
+ * outputs here, not inputs (mid_dtype is an input with FD_STEP_CALLER_PARTIALS).  params->max_kv_len (rounded up to
+ * 1024 tokens, so that a growing batch does not re-plan at every step) replaces the block table's capacity as the
+ * longest sequence to plan for.  Returns 0 or a negative fd_status.  No counterpart in the reference.
+ */
+FD_API int fd_plan_decode(const fd_params* params, int32_t batch, int32_t num_extra, int32_t flags,
+                          fd_launch_plan* plan);
+
+/* fd_plan_decode(...).workspace_bytes, or a negative fd_status: what fd_decode_planned needs for this shape. */
+FD_API int64_t fd_workspace_bytes(const fd_params* params, int32_t batch, int32_t num_extra, int32_t flags);
+
+/*
+ * Every argument of a planned decode step in one block, so that a binding can keep it between steps and touch only
+ * what changed (the reference's wrappers marshal two dozen arguments per launch, flash_decode.py:788-844).
+ */
+typedef struct fd_decode_args {
+  const void* q;              /* [batch, Hq, D]                                                                     */
+  const void* k_cache;        /* [num_pages, P, Hkv, D]                                                             */
+  const void* v_cache;
+  void* workspace;            /* at least fd_workspace_bytes(...) bytes, 256-byte aligned, the caller's; its contents
+                                 mean nothing between calls; calls that may overlap need one each                    */
+  int64_t workspace_bytes;
+  void* out;                  /* [batch, Hq, Dv] (+ 1 column with FD_COMBINE_SPLIT_LSE)                              */
+  float* lse_out;             /* NULL or fp32 [batch, Hq]                                                            */
+  const int32_t* block_table;
+  const int32_t* kv_lens;
+  const int32_t* seq_order;   /* NULL: the library ranks the work itself where that pays; else an order the caller
+                                 computed (fd_schedule, fd_schedule_items with the plan's split fields, fd_kv_append),
+                                 params.seq_order_items / seq_order_lens describing it                              */
+  const void* extra_out;      /* as for fd_combine                                                                   */
+  const float* extra_lse;
+  int64_t stride_q_bs, stride_q_h, stride_k_tok, stride_k_h, stride_v_tok, stride_v_h;
+  int64_t stride_table_bs, stride_obs, stride_oh;
+  float sm_scale;
+  int32_t batch;
+  int32_t combine_mode;       /* FD_COMBINE_SPLIT or FD_COMBINE_SPLIT_LSE                                            */
+  int32_t num_extra;
+  int32_t flags;              /* fd_step_flags: FD_STEP_EXACT_SPLITS, FD_STEP_SCHEDULE, FD_STEP_NO_ORDER              */
+  fd_params params;           /* num_splits is the hint described at fd_plan_decode                                  */
+} fd_decode_args;
+
+/*
+ * One decode step as the library plans it: what gqa_fwd_batch_decode / _intra_rank / _persistent
+ * (flash_decode.py:763-844, 847-928, 931-1005) do when the caller passes no output_split -- the wrappers there pick
+ * 32 splits, allocate the partials and launch split and combine; here the library picks the plan of fd_plan_decode,
+ * keeps partials, LSEs and the issue order in `workspace`, and enqueues the scheduling launch (if the plan has one),
+ * the split kernel and the combine kernel (unless the plan is direct).  The result is the same for every plan.
+ * Returns FD_ERR_INVALID_ARG when the workspace is missing, misaligned or too small (the message names the size).
+ */
+FD_API int fd_decode_planned(void* stream, const fd_decode_args* args);
 
 /*
  * fd_decode for callers that cannot allocate device memory -- code under HIP graph capture, tight serving

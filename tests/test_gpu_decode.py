@@ -944,11 +944,12 @@ def test_item_schedule_matches_oracle_and_is_a_permutation(fd, capacity, kind, b
     # the raw scheduler: a permutation of all (sequence, range) pairs, non-empty ranges first and largest first
     fk = __import__("importlib").import_module("triton-distributed_amd.kernels.flash_decode")
     g = wl.to(DEV)
-    S, adapt = fk.plan_decode(g.q, g.k_cache, g.block_table, -1, k_scale=g.k_scale, v_scale=g.v_scale)
+    plan = fk.decode_plan(g.q, g.k_cache, g.block_table, -1, fp8=g.k_scale is not None)
+    S, adapt, align = plan.num_splits, plan.split_adapt, plan.split_align
     if S == 1 or adapt == 0:
         return
     p = fk._make_params(g.q, g.k_cache, g.block_table, S, 0.0, 0, 0, g.k_scale, g.v_scale, "auto", 0, None,
-                        fk.SPLIT_ALIGN, adapt)
+                        align, adapt)
     items = fk.item_order_buffer(batch, S, DEV)
     fd._lib.check(fd.load_library().fd_schedule_items(None, g.kv_lens.data_ptr(), batch, items.data_ptr(), byref(p)))
     torch.cuda.synchronize()
@@ -959,7 +960,7 @@ def test_item_schedule_matches_oracle_and_is_a_permutation(fd, capacity, kind, b
 
     def per(n):   # the library's range rule (include/flash_decode.h, fd_params.split_adapt)
         v = max(-(-n // S), min(-(-n // adapt), min(max(-(-n // 8), 1024), 4096)))
-        return -(-v // fk.SPLIT_ALIGN) * fk.SPLIT_ALIGN
+        return -(-v // align) * align
     busy = [per(lens[b]) * s < lens[b] for b, s in zip(seq, rng_)]
     n_busy = sum(busy)
     assert all(busy[:n_busy]) and not any(busy[n_busy:])

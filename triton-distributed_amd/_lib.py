@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libflash_decode_gfx950.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-FD_ABI_VERSION = 2
+FD_ABI_VERSION = 3
 
 # fd_dtype
 FD_F32, FD_F16, FD_BF16, FD_FP8_E4M3 = 0, 1, 2, 3
@@ -24,8 +24,13 @@ FD_PATH_AUTO, FD_PATH_VALU, FD_PATH_MFMA = 0, 1, 2
 # fd_combine_mode
 FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_COMBINE_RANK = 0, 1, 2
 FD_NOALLOC_SCRATCH_BYTES = 16 << 20   # static partial workspace of fd_decode_noalloc
+# fd_step_flags
+FD_STEP_EXACT_SPLITS, FD_STEP_SCHEDULE, FD_STEP_NO_ORDER, FD_STEP_FUSED, FD_STEP_LSE_TWICE = 1, 2, 4, 8, 16
+FD_STEP_CALLER_PARTIALS, FD_STEP_ORDER_FROM_APPEND = 32, 64
+# fd_order_kind
+FD_ORDER_NONE, FD_ORDER_SEQUENCES, FD_ORDER_ITEMS = 0, 1, 2
 
-EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_decode_noalloc", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
+EXPORTED_SYMBOLS = ("fd_split_kv", "fd_combine", "fd_decode", "fd_plan_decode", "fd_workspace_bytes", "fd_decode_planned", "fd_decode_noalloc", "fd_schedule", "fd_schedule_items", "fd_plan_splits", "fd_plan_min_splits",
                     "fd_kv_append",
                     "fd_last_error", "fd_abi_version", "fd_build_id")
 
@@ -57,6 +62,30 @@ class FdParams(Structure):
         ("max_kv_len", c_int32),
         ("seq_order_items", c_int32),
         ("v_head_dim", c_int32),
+    ]
+
+
+class FdLaunchPlan(Structure):
+    """Mirror of ``struct fd_launch_plan``."""
+    _fields_ = [
+        ("num_splits", c_int32), ("split_adapt", c_int32), ("split_align", c_int32), ("mid_dtype", c_int32),
+        ("direct", c_int32), ("order_kind", c_int32), ("mfma", c_int32), ("tile", c_int32),
+        ("waves_per_head", c_int32), ("members", c_int32), ("chunk", c_int32), ("head_block", c_int32),
+        ("grid", c_int32 * 3), ("store_through", c_int32), ("max_kv_len", c_int32), ("reserved", c_int32),
+        ("partial_bytes", c_int64), ("lse_bytes", c_int64), ("order_bytes", c_int64), ("workspace_bytes", c_int64),
+    ]
+
+
+class FdDecodeArgs(Structure):
+    """Mirror of ``struct fd_decode_args``."""
+    _fields_ = [
+        ("q", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p), ("workspace", c_void_p),
+        ("workspace_bytes", c_int64), ("out", c_void_p), ("lse_out", c_void_p), ("block_table", c_void_p),
+        ("kv_lens", c_void_p), ("seq_order", c_void_p), ("extra_out", c_void_p), ("extra_lse", c_void_p),
+        ("stride_q_bs", c_int64), ("stride_q_h", c_int64), ("stride_k_tok", c_int64), ("stride_k_h", c_int64),
+        ("stride_v_tok", c_int64), ("stride_v_h", c_int64), ("stride_table_bs", c_int64), ("stride_obs", c_int64),
+        ("stride_oh", c_int64), ("sm_scale", c_float), ("batch", c_int32), ("combine_mode", c_int32),
+        ("num_extra", c_int32), ("flags", c_int32), ("params", FdParams),
     ]
 
 
@@ -103,6 +132,12 @@ def load_library(path: str = None) -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
         c_int32, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, c_void_p, c_int32, c_void_p, c_void_p,
         c_int32, c_void_p, POINTER(FdParams)]
+    lib.fd_plan_decode.restype = c_int32
+    lib.fd_plan_decode.argtypes = [POINTER(FdParams), c_int32, c_int32, c_int32, POINTER(FdLaunchPlan)]
+    lib.fd_workspace_bytes.restype = c_int64
+    lib.fd_workspace_bytes.argtypes = [POINTER(FdParams), c_int32, c_int32, c_int32]
+    lib.fd_decode_planned.restype = c_int32
+    lib.fd_decode_planned.argtypes = [c_void_p, POINTER(FdDecodeArgs)]
     lib.fd_decode_noalloc.restype = c_int32
     lib.fd_decode_noalloc.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int32,

@@ -214,12 +214,21 @@ struct FusedTail {          // what the fused combine needs on top of the split 
 // Largest dynamic LDS a workgroup may ask for on gfx950 (160 KB per CU).
 constexpr size_t kMaxLds = 160 * 1024;
 
+// What a launch of the split kernel looks like (fd_launch_plan reports it).
+struct LaunchShape {
+  int mfma, tile, waves_per_head, members, chunk, head_block, store_through;
+  unsigned grid[3];
+};
+
+// shape_only: the launch shape is reported there and nothing is launched (the pointers are only checked, never
+// dereferenced on the host, so a planner may pass stand-ins).
 int split_impl(const char* fn, void* stream, const void* q, const void* k_cache, const void* v_cache,
                void* out_split, float* lse_split, float sm_scale, const int32_t* block_table,
                const int32_t* kv_lens, int32_t batch, int64_t stride_q_bs, int64_t stride_q_h, int64_t stride_k_tok,
                int64_t stride_k_h, int64_t stride_v_tok, int64_t stride_v_h, int64_t stride_o_bs, int64_t stride_o_h,
                int64_t stride_o_split, int64_t stride_table_bs, const int32_t* seq_order, const fd_params* p,
-               const FusedTail* tail, bool* fused, bool no_lse = false, bool skip_empty = false) {
+               const FusedTail* tail, bool* fused, bool no_lse = false, bool skip_empty = false,
+               LaunchShape* shape_only = nullptr) {
   if (fused) *fused = false;
   if (!p) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
   if (!q || !k_cache || !v_cache || !out_split || !block_table || !kv_lens)
@@ -482,6 +491,18 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     }
   }
 
+  if (shape_only) {
+    shape_only->mfma = use_mfma ? 1 : 0;
+    shape_only->tile = tile;
+    shape_only->waves_per_head = a.nsub;
+    shape_only->members = a.hpw;
+    shape_only->chunk = a.chunk;
+    shape_only->head_block = a.hbsz;
+    shape_only->store_through = a.store_through;
+    const dim3 grid = fd_split_grid(a);
+    shape_only->grid[0] = grid.x; shape_only->grid[1] = grid.y; shape_only->grid[2] = grid.z;
+    return FD_OK;
+  }
   int rc;
   if (use_mfma && kv_fp8 && D == 256) {
     rc = fd_launch_split_mfma_fp8_d256((hipStream_t)stream, a, p->q_dtype, waves, a.soft_cap > 0.f);
@@ -904,6 +925,236 @@ int fd_schedule(void* stream, const int32_t* kv_lens, int32_t batch, int32_t* se
   int rc = fd_launch_schedule((hipStream_t)stream, kv_lens, batch, seq_order);
   if (rc != FD_OK) return fail(rc, "fd_schedule: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return FD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The launch policy of a decode step whose partials the caller does not see (fd_plan_decode / fd_decode_planned).
+
+namespace {
+
+constexpr int kDefaultSplits = 32;        // flash_decode.py:779
+constexpr int kPlannedSplitAlign = 64;    // tokens: the largest tile of the split kernels
+constexpr int kMaxAutoSplits = 256;       // upper bound of the library's own choice
+constexpr int64_t kPartials16BitFromBytes = 4 << 20;   // fp32 partials of a planned step from which on they take the output's 16-bit type
+// Largest batch the step schedules as (sequence, range) items of its own accord; beyond it the item list costs more
+// than it gains over the per-sequence order (256 ragged sequences of up to 8192 tokens: 650 against 640 us, 160 of
+// them: 426 against 435 us)
+constexpr int kItemsUpToBatch = 192;
+// From this batch size on a step that was not asked to schedule ranks its sequences all the same (one launch of
+// 3.5 us): a batch that large is ragged in practice and runs 4 - 15 % faster longest first (256 sequences of up to 2048
+// tokens: 187 against 159 us, 72 of up to 8192 tokens 213 against 196 us); a uniform one loses the launch.
+constexpr int kAutoOrderFromBatch = 64;
+constexpr int kAutoOrderMinCapacity = 1024;   // ... unless no sequence can be longer than a range
+constexpr int kMaxSeqOrderBatch = 4096;       // sequences fd_schedule ranks for a step
+constexpr int kAppendOrderFromBatch = 16;     // an order that costs no launch (the append computes it) pays earlier
+
+int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
+
+// Upper bound of the split count when the partials stay inside the library.  The caller's count is a hint there, not a
+// limit -- the result does not depend on it, and the reference's 32 were chosen for contexts of a few thousand tokens:
+// a single sequence of 131072 tokens on 8 KV heads runs 5 % faster with 64.
+int split_bound(int hint, int64_t tokens) {
+  int64_t own = tokens / 512;
+  if (own > kMaxAutoSplits) own = kMaxAutoSplits;
+  if (own < kDefaultSplits) own = kDefaultSplits;
+  return hint > own ? hint : (int)own;
+}
+
+struct StepPlan {
+  fd_params p;          // the parameters fd_decode / fd_split_kv / fd_combine / fd_schedule_items run the step with
+  int direct, order_kind;
+  int64_t partial_bytes, lse_bytes, order_bytes, lse_off, order_off, total;
+  int64_t so_b, so_h, so_s;   // element strides of the partials in the workspace
+};
+
+int plan_step(const char* fn, const fd_params* in, int32_t batch, int32_t num_extra, int32_t flags,
+              bool caller_order, StepPlan* sp) {
+  if (!in) return fail(FD_ERR_INVALID_ARG, "%s: params is NULL", fn);
+  if (batch <= 0 || num_extra < 0) return fail(FD_ERR_INVALID_ARG, "%s: batch %d, num_extra %d", fn, batch, num_extra);
+  if (in->q_heads <= 0 || in->kv_heads <= 0 || in->q_heads % in->kv_heads != 0 || in->page_size <= 0 ||
+      in->max_pages_per_seq <= 0)
+    return fail(FD_ERR_INVALID_ARG, "%s: q_heads %d, kv_heads %d, page_size %d, max_pages_per_seq %d", fn, in->q_heads,
+                in->kv_heads, in->page_size, in->max_pages_per_seq);
+  const int Dv = v_dim(in);
+  if (Dv != 64 && Dv != 128 && Dv != 256) return fail(FD_ERR_UNSUPPORTED, "%s: v_head_dim %d (64/128/256)", fn, Dv);
+  const bool exact = (flags & (FD_STEP_EXACT_SPLITS | FD_STEP_CALLER_PARTIALS)) != 0;
+  const bool caller_partials = (flags & FD_STEP_CALLER_PARTIALS) != 0;
+  const bool fused = (flags & FD_STEP_FUSED) != 0;
+  StepPlan& r = *sp;
+  memset(&r, 0, sizeof(r));
+  r.p = *in;
+  const int64_t capacity = (int64_t)in->max_pages_per_seq * in->page_size;
+  // the host-side length hint: rounded up to 1024 tokens, so that a growing batch does not re-plan at every step
+  int64_t hint = 0;
+  if (in->max_kv_len > 0 && in->max_kv_len < capacity) {
+    hint = ((int64_t)in->max_kv_len + 1023) / 1024 * 1024;
+    if (hint >= capacity) hint = 0;
+  }
+  r.p.max_kv_len = (int32_t)hint;
+  r.p.seq_order_items = caller_order ? in->seq_order_items : 0;
+  if (!caller_order) r.p.seq_order_lens = nullptr;
+  if (exact) {
+    r.p.num_splits = in->num_splits > 0 ? in->num_splits : kDefaultSplits;
+    r.p.split_adapt = 0;
+    r.p.split_align = caller_partials ? 0 : kPlannedSplitAlign;
+  } else {
+    // nobody looks at the partials: the library chooses the split count.  The grid has num_splits slots per
+    // sequence; a sequence uses as many as its own length asks for (split_adapt).
+    r.p.num_splits = split_bound(in->num_splits, hint ? hint : capacity);
+    r.p.split_adapt = 0;
+    r.p.split_align = kPlannedSplitAlign;
+    const int s = fd_plan_splits(&r.p, batch);
+    if (s < 0) return s;
+    const int k = fd_plan_min_splits(&r.p, batch);
+    if (k < 0) return k;
+    r.p.num_splits = s;
+    r.p.split_adapt = k;
+  }
+  const int S = r.p.num_splits;
+  const int64_t rows = (int64_t)batch * in->q_heads * S;
+  r.direct = S == 1 && num_extra == 0 && !fused && !caller_partials && !(flags & FD_STEP_LSE_TWICE);
+  // Element type of the partials (the LSEs are always fp32, in their own buffer).  Planned splits are few and long:
+  // fp32, unless there are kPartials16BitFromBytes of them or more (many query heads per KV head, large batches).
+  // Those, and the partials of a caller who insists on an exact count, take the output's precision when that is
+  // 16-bit -- what the reference's intra-rank wrapper allocates (flash_decode.py:867-868; the plain one fp16 whatever
+  // the inputs, :783-784): megabytes that the split kernel writes at its very end and the combine reads back.
+  if (!caller_partials) {
+    static const int64_t from_bytes = env_int("FD_PARTIALS_16BIT_FROM_BYTES") > 0 ? env_int("FD_PARTIALS_16BIT_FROM_BYTES")
+                                                                                   : kPartials16BitFromBytes;
+    const bool out16 = in->out_dtype == FD_F16 || in->out_dtype == FD_BF16;
+    r.p.mid_dtype = !fused && out16 && (exact || rows * Dv * 4 >= from_bytes) ? in->out_dtype : FD_F32;
+  }
+  // The issue order the step computes itself.
+  r.order_kind = FD_ORDER_NONE;
+  if (!caller_order && !(flags & FD_STEP_NO_ORDER) && batch > 1) {
+    const bool free_order = (flags & FD_STEP_ORDER_FROM_APPEND) && batch >= kAppendOrderFromBatch;
+    const bool scheduled = (flags & FD_STEP_SCHEDULE) || free_order;
+    const bool items = scheduled && S > 1 && !fused && batch <= kItemsUpToBatch;
+    const bool ranked = scheduled || (batch >= kAutoOrderFromBatch && capacity >= kAutoOrderMinCapacity);
+    if (items) {
+      r.order_kind = FD_ORDER_ITEMS;
+      r.p.seq_order_items = 1;
+    } else if (ranked && batch <= kMaxSeqOrderBatch) {
+      r.order_kind = FD_ORDER_SEQUENCES;
+    }
+  }
+  const int msz = dtype_size(r.p.mid_dtype);
+  if (!msz || r.p.mid_dtype == FD_FP8_E4M3) return fail(FD_ERR_UNSUPPORTED, "%s: mid_dtype %d", fn, r.p.mid_dtype);
+  r.so_s = caller_partials ? Dv + 1 : Dv;
+  r.so_h = (int64_t)S * r.so_s;
+  r.so_b = (int64_t)in->q_heads * r.so_h;
+  r.partial_bytes = caller_partials ? 0 : rows * Dv * msz;
+  r.lse_bytes = caller_partials ? 0 : rows * 4;
+  r.order_bytes = r.order_kind == FD_ORDER_ITEMS ? 2 * (int64_t)batch * S * 4
+                  : r.order_kind == FD_ORDER_SEQUENCES ? (int64_t)batch * 4 : 0;
+  r.lse_off = align256(r.partial_bytes);
+  r.order_off = r.lse_off + align256(r.lse_bytes);
+  r.total = r.order_off + align256(r.order_bytes);
+  return FD_OK;
+}
+
+}  // namespace
+
+int fd_plan_decode(const fd_params* params, int32_t batch, int32_t num_extra, int32_t flags, fd_launch_plan* plan) {
+  const char* fn = "fd_plan_decode";
+  if (!plan) return fail(FD_ERR_INVALID_ARG, "%s: plan is NULL", fn);
+  StepPlan sp;
+  if (int rc = plan_step(fn, params, batch, num_extra, flags, false, &sp)) return rc;
+  memset(plan, 0, sizeof(*plan));
+  plan->num_splits = sp.p.num_splits;
+  plan->split_adapt = sp.p.split_adapt;
+  plan->split_align = sp.p.split_align;
+  plan->mid_dtype = sp.p.mid_dtype;
+  plan->direct = sp.direct;
+  plan->order_kind = sp.order_kind;
+  plan->partial_bytes = sp.partial_bytes;
+  plan->lse_bytes = sp.lse_bytes;
+  plan->order_bytes = sp.order_bytes;
+  plan->workspace_bytes = sp.total;
+  plan->max_kv_len = sp.p.max_kv_len;
+  // The launch shape, for contiguous caches and a contiguous query; the pointers below are stand-ins that are
+  // checked for alignment only.
+  void* const fake = reinterpret_cast<void*>((uintptr_t)1 << 20);
+  fd_params p = sp.p;
+  float one = 1.f;   // stand-in for fp8 scales (checked for presence only)
+  if (p.kv_dtype == FD_FP8_E4M3) {
+    if (!p.k_scale) p.k_scale = &one;
+    if (!p.v_scale) p.v_scale = &one;
+  }
+  if (p.num_pages <= 0) p.num_pages = p.max_pages_per_seq;
+  const int Dv = v_dim(&p);
+  const bool caller_partials = (flags & FD_STEP_CALLER_PARTIALS) != 0;
+  const bool skip_empty = !sp.direct && p.split_adapt > 0 && p.split_adapt < p.num_splits &&
+                          p.num_splits > kCombineSmallMax && !(flags & FD_STEP_FUSED);
+  int32_t ticket = 0;
+  FusedTail tail;
+  tail.tickets = (flags & FD_STEP_FUSED) ? &ticket : nullptr;
+  tail.num_extra = num_extra;
+  bool fused = false;
+  if (sp.direct) p.mid_dtype = p.out_dtype;
+  LaunchShape ls;
+  memset(&ls, 0, sizeof(ls));
+  const int32_t* order = sp.order_kind != FD_ORDER_NONE ? (const int32_t*)fake : nullptr;
+  int rc = split_impl(fn, nullptr, fake, fake, fake, fake, caller_partials ? nullptr : (float*)fake, 1.f,
+                      (const int32_t*)fake, (const int32_t*)fake, batch, (int64_t)p.q_heads * p.head_dim, p.head_dim,
+                      (int64_t)p.kv_heads * p.head_dim, p.head_dim, (int64_t)p.kv_heads * Dv, Dv,
+                      sp.direct ? (int64_t)p.q_heads * Dv : sp.so_b, sp.direct ? Dv : sp.so_h, sp.direct ? 0 : sp.so_s,
+                      p.max_pages_per_seq, order, &p, &tail, &fused, false, skip_empty, &ls);
+  if (rc != FD_OK) return rc;
+  plan->mfma = ls.mfma;
+  plan->tile = ls.tile;
+  plan->waves_per_head = ls.waves_per_head;
+  plan->members = ls.members;
+  plan->chunk = ls.chunk;
+  plan->head_block = ls.head_block;
+  plan->store_through = ls.store_through;
+  for (int i = 0; i < 3; ++i) plan->grid[i] = (int32_t)ls.grid[i];
+  return FD_OK;
+}
+
+int64_t fd_workspace_bytes(const fd_params* params, int32_t batch, int32_t num_extra, int32_t flags) {
+  StepPlan sp;
+  if (int rc = plan_step("fd_workspace_bytes", params, batch, num_extra, flags, false, &sp)) return rc;
+  return sp.total;
+}
+
+int fd_decode_planned(void* stream, const fd_decode_args* a) {
+  const char* fn = "fd_decode_planned";
+  if (!a) return fail(FD_ERR_INVALID_ARG, "%s: args is NULL", fn);
+  if (a->batch == 0) return FD_OK;
+  if (a->flags & ~(FD_STEP_EXACT_SPLITS | FD_STEP_SCHEDULE | FD_STEP_NO_ORDER))
+    return fail(FD_ERR_INVALID_ARG, "%s: flags 0x%x (FD_STEP_EXACT_SPLITS | FD_STEP_SCHEDULE | FD_STEP_NO_ORDER)", fn,
+                a->flags);
+  if (a->combine_mode != FD_COMBINE_SPLIT && a->combine_mode != FD_COMBINE_SPLIT_LSE)
+    return fail(FD_ERR_INVALID_ARG, "%s: combine_mode %d (FD_COMBINE_SPLIT or FD_COMBINE_SPLIT_LSE)", fn, a->combine_mode);
+  if (!a->kv_lens) return fail(FD_ERR_INVALID_ARG, "%s: NULL tensor pointer", fn);
+  const int lse_twice = a->combine_mode == FD_COMBINE_SPLIT_LSE && a->lse_out ? FD_STEP_LSE_TWICE : 0;
+  StepPlan sp;
+  if (int rc = plan_step(fn, &a->params, a->batch, a->num_extra, a->flags | lse_twice, a->seq_order != nullptr, &sp))
+    return rc;
+  const bool need_ws = !sp.direct || sp.order_kind != FD_ORDER_NONE;
+  char* ws = (char*)a->workspace;
+  if (need_ws) {
+    if (!ws || (reinterpret_cast<uintptr_t>(ws) & 255u) || a->workspace_bytes < sp.total)
+      return fail(FD_ERR_INVALID_ARG,
+                  "%s: the step needs a 256-byte aligned workspace of %lld bytes (fd_workspace_bytes), got %p with %lld",
+                  fn, (long long)sp.total, (void*)ws, (long long)a->workspace_bytes);
+  }
+  const int32_t* order = a->seq_order;
+  if (sp.order_kind == FD_ORDER_ITEMS) {
+    int32_t* items = (int32_t*)(ws + sp.order_off);
+    if (int rc = fd_schedule_items(stream, a->kv_lens, a->batch, items, &sp.p)) return rc;
+    order = items;
+  } else if (sp.order_kind == FD_ORDER_SEQUENCES) {
+    int32_t* seq = (int32_t*)(ws + sp.order_off);
+    if (int rc = fd_schedule(stream, a->kv_lens, a->batch, seq)) return rc;
+    order = seq;
+  }
+  return fd_decode(stream, a->q, a->k_cache, a->v_cache, sp.direct ? nullptr : ws,
+                   sp.direct ? nullptr : (float*)(ws + sp.lse_off), a->out, a->lse_out, a->sm_scale, a->block_table,
+                   a->kv_lens, a->batch, a->stride_q_bs, a->stride_q_h, a->stride_k_tok, a->stride_k_h, a->stride_v_tok,
+                   a->stride_v_h, sp.so_b, sp.so_h, sp.so_s, a->stride_table_bs, a->stride_obs, a->stride_oh, order,
+                   a->combine_mode, a->extra_out, a->extra_lse, a->num_extra, nullptr, &sp.p);
 }
 
 }  // extern "C"

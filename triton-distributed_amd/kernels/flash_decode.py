@@ -15,15 +15,19 @@ Keyword-only additions that the reference does not have (all default off):
   extra_partials  (out [E,B,Hq,Dv], lse [E,B,Hq] fp32): further partials merged by
                   the combine, standing in for what other sequence-parallel ranks
                   would contribute
-  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (batches of
-                  ``AUTO_ORDER_FROM_BATCH`` = 64 sequences or more are ranked by the wrapper itself when none is given)
+  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (batches of 64 sequences or
+                  more are ranked by the step itself when none is given; ``auto_order=False`` switches that off)
   seq_order_lens  int32 [B], with ``seq_order``: ``kv_lens[seq_order]`` (``rope_kv_append`` writes both), which
                   saves a workgroup one dependent load before it can start
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
   plan_splits     True (default): when ``output_split`` is not supplied, ``kv_split`` is a hint and the library
-                  uses ``fd_plan_splits`` splits (same result; usually fewer -- fewer workgroup prologues and
-                  partials --, more for block tables of more than 16384 tokens); False: exactly ``kv_split`` splits.  With a caller-supplied
-                  ``output_split`` the split count and ranges are always the reference's.
+                  plans the step (``fd_decode_planned``: same result; usually fewer splits -- fewer workgroup prologues
+                  and partials --, more for block tables of more than 16384 tokens); False: exactly ``kv_split``
+                  splits.  With a caller-supplied ``output_split`` the split count and ranges are always the
+                  reference's.
+  workspace       the reference's positional argument; a contiguous GPU tensor of at least ``workspace_bytes(...)``
+                  bytes on a 256-byte boundary holds partials, LSEs and issue order of a planned step, which then
+                  allocates nothing; anything else is ignored, as in the reference
   no_alloc        True: the split partials live in the library's static device array (``fd_decode_noalloc``, at most
                   16 MiB of them) and the call allocates nothing -- for steps captured into a HIP graph or run where
                   allocation is not allowed; needs ``output_combine``; calls that overlap on one GPU must not share it
@@ -36,27 +40,26 @@ Differences from the reference, on purpose: when ``output_split`` is not
 supplied the partials stay inside the library as ``[B,Hq,S,Dv]`` with the LSEs
 in their own fp32 buffer -- fp32 values, or the output's 16-bit type once there
 are 4 MB of them or the caller insists on exactly ``kv_split`` splits
-(``internal_partial_dtype``; the reference allocates fp16 ``[B,Hq,S,Dv+1]``,
+(``fd_plan_decode`` decides; the reference allocates fp16 ``[B,Hq,S,Dv+1]``,
 :783-784); the default ``output_combine`` has the query's dtype (the reference
 hard-codes fp16, :785, which is the same thing for the fp16 inputs its tests
 use).
 """
 from __future__ import annotations
 
-import os
-
 from ctypes import byref
 from typing import Optional
 
 import torch
 
-from .._lib import (FD_BF16, FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F16, FD_F32, FD_NOALLOC_SCRATCH_BYTES, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
-                    FdParams, check, fd_dtype_of, load_library, stream_handle)
+from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F32, FD_NOALLOC_SCRATCH_BYTES,
+                    FD_ORDER_ITEMS, FD_ORDER_SEQUENCES, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
+                    FD_STEP_CALLER_PARTIALS, FD_STEP_EXACT_SPLITS, FD_STEP_FUSED, FD_STEP_LSE_TWICE, FD_STEP_NO_ORDER,
+                    FD_STEP_SCHEDULE, FdDecodeArgs, FdLaunchPlan, FdParams, check, fd_dtype_of, load_library,
+                    stream_handle)
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
 DEFAULT_KV_SPLITS = 32  # flash_decode.py:779
-SPLIT_ALIGN = 64        # tokens: the largest tile of the split kernels
-MAX_AUTO_KV_SPLITS = 256  # upper bound of the library's own choice (kv_split == -1, internal partials)
 
 
 def get_split_kv_algo_info(q_heads, kv_heads, q_head_dim, v_head_dim, page_size, split_kv=32, soft_cap=0.0):
@@ -87,37 +90,6 @@ def get_combine_kv_algo_info(split_kv=32, v_head_dim=128, block_dv=512):
 get_triton_combine_kv_algo_info = get_combine_kv_algo_info
 
 
-def auto_split_bound(capacity: int) -> int:
-    """Upper bound of the split count when the caller leaves it to the library (``kv_split == -1`` and no
-    ``output_split``): the reference's 32 (flash_decode.py:779), more for block tables of more than 16384 tokens."""
-    return max(DEFAULT_KV_SPLITS, min(MAX_AUTO_KV_SPLITS, capacity // 512))
-
-
-def split_bound(kv_split: int, capacity: int) -> int:
-    """Most splits a step may be planned with when its partials stay inside the library.  The caller's ``kv_split`` is
-    a hint there, not a limit -- the result does not depend on the count, and the reference's 32 were chosen for
-    contexts of a few thousand tokens: a single sequence of 131072 tokens on 8 KV heads runs 5 % faster with 64."""
-    auto = auto_split_bound(capacity)
-    return auto if kv_split == -1 else max(kv_split, auto)
-
-
-PARTIALS_16BIT_FROM_BYTES = int(os.environ.get("FD_PARTIALS_16BIT_FROM_BYTES", 4 << 20))
-
-
-def internal_partial_dtype(out_dtype, plan_splits, fuse_combine, partial_elems=0):
-    """Element type of the partials when they stay inside the library (the LSEs are always fp32, in their own
-    buffer).  Planned splits are few and long: fp32, unless there are ``PARTIALS_16BIT_FROM_BYTES`` of them or more
-    (many query heads per KV head, large batches).  Those, and the partials of a caller who insists on exactly
-    ``kv_split`` splits (``plan_splits=False``), take the output's precision when that is 16-bit -- what the
-    reference's intra-rank wrapper allocates (flash_decode.py:867-868; the plain one fp16 whatever the inputs,
-    :783-784): megabytes that the split kernel writes at its very end and the combine reads back."""
-    if fuse_combine or out_dtype not in (torch.float16, torch.bfloat16):
-        return FD_F32
-    if plan_splits and 4 * partial_elems < PARTIALS_16BIT_FROM_BYTES:
-        return FD_F32
-    return FD_F16 if out_dtype == torch.float16 else FD_BF16
-
-
 def _require_cuda(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -136,9 +108,33 @@ def schedule_sequences(kv_lens: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
+def _fill_params(t: FdParams, q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, fp8, path,
+                 waves_per_block, split_align, split_adapt, seq_order_items, max_kv_len, v_head_dim):
+    t.q_heads = q.shape[1]
+    t.kv_heads = k_cache.shape[2]
+    t.head_dim = q.shape[2]
+    t.v_head_dim = v_head_dim if v_head_dim and v_head_dim != q.shape[2] else 0
+    t.page_size = k_cache.shape[1]
+    t.num_splits = kv_split
+    t.num_pages = k_cache.shape[0]
+    t.max_pages_per_seq = block_table.shape[1]
+    t.q_dtype = fd_dtype_of(q)
+    t.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=fp8)
+    t.mid_dtype = mid_dtype
+    t.out_dtype = out_dtype
+    t.soft_cap = float(soft_cap or 0.0)
+    t.path = _PATHS[path]
+    t.waves_per_block = waves_per_block
+    t.split_align = split_align
+    t.split_adapt = split_adapt
+    t.seq_order_items = seq_order_items
+    t.max_kv_len = int(max_kv_len or 0)
+
+
 def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale, v_scale, path,
                  waves_per_block, seq_order_lens=None, split_align=0, split_adapt=0, seq_order_items=0,
                  max_kv_len=0, v_head_dim=0) -> FdParams:
+    """``fd_params`` of an explicit call (``fd_decode`` / ``fd_split_kv`` / ``fd_combine``): every field as given."""
     # the scalar fields are the same from step to step: filled once per combination, copied per call
     v_head_dim = v_head_dim or q.shape[2]
     key = (q.shape, k_cache.shape, block_table.shape[1], q.dtype, k_cache.dtype, k_scale is not None, kv_split, soft_cap,
@@ -147,25 +143,8 @@ def _make_params(q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dty
     template = _PARAMS_CACHE.get(key)
     if template is None:
         t = FdParams()
-        t.q_heads = q.shape[1]
-        t.kv_heads = k_cache.shape[2]
-        t.head_dim = q.shape[2]
-        t.v_head_dim = v_head_dim if v_head_dim != q.shape[2] else 0
-        t.page_size = k_cache.shape[1]
-        t.num_splits = kv_split
-        t.num_pages = k_cache.shape[0]
-        t.max_pages_per_seq = block_table.shape[1]
-        t.q_dtype = fd_dtype_of(q)
-        t.kv_dtype = fd_dtype_of(k_cache, fp8_bytes=k_scale is not None)
-        t.mid_dtype = mid_dtype
-        t.out_dtype = out_dtype
-        t.soft_cap = float(soft_cap or 0.0)
-        t.path = _PATHS[path]
-        t.waves_per_block = waves_per_block
-        t.split_align = split_align
-        t.split_adapt = split_adapt
-        t.seq_order_items = seq_order_items
-        t.max_kv_len = max_kv_len
+        _fill_params(t, q, k_cache, block_table, kv_split, soft_cap, mid_dtype, out_dtype, k_scale is not None, path,
+                     waves_per_block, split_align, split_adapt, seq_order_items, max_kv_len, v_head_dim)
         if len(_PARAMS_CACHE) > 4096:
             _PARAMS_CACHE.clear()
         template = _PARAMS_CACHE[key] = bytes(t)
@@ -182,49 +161,60 @@ _PARAMS_CACHE = {}   # fd_params images by their scalar fields
 
 MAX_ITEM_BATCH = 1024       # sequences fd_schedule_items ranks in one launch
 MAX_FUSED_ITEM_BATCH = 256  # ... and fd_kv_append in its trailing workgroup
-MAX_SEQ_ORDER_BATCH = 4096  # sequences the scheduled variant ranks with fd_schedule where items do not apply
-# Largest batch the wrappers schedule as (sequence, range) items of their own accord; beyond it the item list costs
-# more than it gains over the per-sequence order (256 ragged sequences of up to 8192 tokens: 650 against 640 us,
-# 160 of them: 426 against 435 us)
-ITEMS_UP_TO_BATCH = 192
-# From this batch size on the plain wrappers rank the sequences as well (one launch of 3.5 us): a batch that large is
-# ragged in practice and runs 4 - 15 % faster longest first (256 sequences of up to 2048 tokens: 187 against 159 us,
-# 72 of up to 8192 tokens 213 against 196 us), a uniform one loses the launch.  0 switches it off; callers that pass
-# ``seq_order`` / ``item_order`` are not touched.
-AUTO_ORDER_FROM_BATCH = 64
 
 
-def _hint(max_kv_len, capacity):
-    """The host-side length hint as the library takes it: 0 = none, else rounded up to a multiple of 1024 tokens so
-    that a growing batch does not re-plan at every step."""
-    if not max_kv_len or max_kv_len >= capacity:
-        return 0
-    return min(capacity, -(-int(max_kv_len) // 1024) * 1024)
+class DecodePlan:
+    """``fd_plan_decode`` for a shape: the library's launch policy as the wrappers see it (read-only)."""
+    __slots__ = ("num_splits", "split_adapt", "split_align", "mid_dtype", "direct", "order_kind", "workspace_bytes",
+                 "max_kv_len", "launch")
+
+    def __init__(self, lp: FdLaunchPlan):
+        self.num_splits, self.split_adapt, self.split_align = lp.num_splits, lp.split_adapt, lp.split_align
+        self.mid_dtype, self.direct, self.order_kind = lp.mid_dtype, bool(lp.direct), lp.order_kind
+        self.workspace_bytes, self.max_kv_len = lp.workspace_bytes, lp.max_kv_len
+        # the launch shape of the split kernel, for tests and reports
+        self.launch = dict(mfma=bool(lp.mfma), tile=lp.tile, waves_per_head=lp.waves_per_head, members=lp.members,
+                           chunk=lp.chunk, head_block=lp.head_block, grid=tuple(lp.grid),
+                           store_through=bool(lp.store_through), partial_bytes=lp.partial_bytes)
+
+
+def decode_plan(q, k_cache, block_table, kv_split=-1, *, flags=0, out_dtype=None, mid_dtype=FD_F32, num_extra=0,
+                fp8=False, path="auto", waves_per_block=0, max_kv_len=None, v_head_dim=0) -> DecodePlan:
+    """The library's plan of a decode step of this shape (``fd_plan_decode``; cached by shape): split count and
+    ranges, type of the partials, whether the step ranks its work first, workspace size, launch shape.  All launch
+    policy lives in the library; the wrappers only carry this out.  ``kv_split`` is the caller's hint (-1: none), or
+    the exact count with ``FD_STEP_EXACT_SPLITS`` / ``FD_STEP_CALLER_PARTIALS``."""
+    out_dt = fd_dtype_of(q) if out_dtype is None else out_dtype
+    hint = -(-max_kv_len // 1024) * 1024 if max_kv_len else 0   # the library plans in steps of 1024 tokens
+    key = (q.shape, k_cache.shape[1:], block_table.shape[1], q.dtype, k_cache.dtype, fp8, kv_split, flags, out_dt,
+           mid_dtype, num_extra, path, waves_per_block, hint, v_head_dim or q.shape[2])
+    plan = _PLAN_CACHE.get(key)
+    if plan is None:
+        lib = load_library()
+        p = FdParams()
+        _fill_params(p, q, k_cache, block_table, kv_split, 0.0, mid_dtype, out_dt, fp8, path, waves_per_block, 0, 0, 0,
+                     hint, v_head_dim)
+        lp = FdLaunchPlan()
+        check(lib.fd_plan_decode(byref(p), q.shape[0], num_extra, flags, byref(lp)))
+        if len(_PLAN_CACHE) > 4096:
+            _PLAN_CACHE.clear()
+        plan = _PLAN_CACHE[key] = DecodePlan(lp)
+    return plan
 
 
 def plan_decode(q, k_cache, block_table, kv_split=-1, *, k_scale=None, v_scale=None, path="auto", waves_per_block=0,
                 max_kv_len=None, v_head_dim=0):
-    """The split plan of a decode step whose partials stay inside the library: ``(num_splits, split_adapt)`` --
-    grid slots per sequence and the ranges every sequence gets however short it is (``fd_plan_splits``,
-    ``fd_plan_min_splits``; cached by shape).  ``kv_split`` is the caller's hint (``split_bound``), -1 leaves it to the library;
-    ``max_kv_len`` an upper bound of the lengths known on the host (else the block table's capacity counts)."""
-    batch, q_heads, q_head_dim = q.shape
-    page_size, kv_heads = k_cache.shape[1], k_cache.shape[2]
-    capacity = block_table.shape[1] * page_size
-    hint = _hint(max_kv_len, capacity)
-    bound = split_bound(kv_split, hint or capacity)
-    key = (batch, q_heads, kv_heads, q_head_dim, page_size, bound, block_table.shape[1], k_cache.dtype,
-           k_scale is not None, path, hint, v_head_dim or q_head_dim)
-    planned = _PLAN_CACHE.get(key)
-    if planned is None:
-        lib = load_library()
-        plan = _make_params(q, k_cache, block_table, bound, 0.0, FD_F32, FD_F32, k_scale, v_scale, path,
-                            waves_per_block, max_kv_len=hint, v_head_dim=v_head_dim)
-        planned = (lib.fd_plan_splits(byref(plan), batch), lib.fd_plan_min_splits(byref(plan), batch))
-        if min(planned) < 0:
-            check(min(planned))
-        _PLAN_CACHE[key] = planned
-    return planned
+    """``(num_splits, split_adapt)`` of a decode step whose partials stay inside the library: grid slots per sequence
+    and the ranges every sequence gets however short it is (see ``decode_plan``)."""
+    plan = decode_plan(q, k_cache, block_table, kv_split, fp8=k_scale is not None, path=path,
+                       waves_per_block=waves_per_block, max_kv_len=max_kv_len, v_head_dim=v_head_dim)
+    return plan.num_splits, plan.split_adapt
+
+
+def workspace_bytes(q, k_cache, block_table, kv_split=-1, **kw) -> int:
+    """Bytes of workspace a planned decode step of this shape uses (``fd_workspace_bytes``): a contiguous GPU tensor of
+    at least that many bytes passed as ``workspace`` makes the step allocation-free.  Keywords as for ``decode_plan``."""
+    return decode_plan(q, k_cache, block_table, kv_split, **kw).workspace_bytes
 
 
 def item_order_buffer(batch, num_splits, device):
@@ -232,110 +222,37 @@ def item_order_buffer(batch, num_splits, device):
     return torch.empty(2 * batch * num_splits, dtype=torch.int32, device=device)
 
 
+_STEP_CACHE = {}   # fd_decode_args images of planned steps by everything but the pointers
+
+
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
             seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
-            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False):
+            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False, auto_order=True):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
-    assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
-    v_head_dim = v_cache.shape[-1]
+    v_shape = v_cache.shape
+    assert page_size == v_shape[1] and kv_heads == v_shape[2] and k_head_dim == q_head_dim
+    v_head_dim = v_shape[3]
     assert q_heads % kv_heads == 0
-    _require_cuda(q, k_cache, v_cache, kv_lens, block_table, output_split, output_combine)
+    if not (q.is_cuda and k_cache.is_cuda and v_cache.is_cuda and kv_lens.is_cuda and block_table.is_cuda):
+        _require_cuda(q, k_cache, v_cache, kv_lens, block_table)
     assert kv_lens.dtype == torch.int32 and block_table.dtype == torch.int32
     q_st, k_st, v_st = q.stride(), k_cache.stride(), v_cache.stride()
-    assert q_st[-1] == 1 and k_st[-1] == 1 and v_st[-1] == 1
+    assert q_st[2] == 1 and k_st[3] == 1 and v_st[3] == 1
     # kv_loc = page * P + slot is a flat token index (flash_decode.py:205-206): the pool must be linear in it
     assert k_st[0] == page_size * k_st[1] and v_st[0] == page_size * v_st[1]
     if (k_scale is None) != (v_scale is None):
         raise RuntimeError("k_scale and v_scale must be given together")
-    num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
-    lib = load_library()
-    hstream = stream_handle(stream, q.device.index)
-
-    # Partials.  Internal ones are fp32 [B,Hq,S,Dv] + LSE [B,Hq,S] addressed by raw pointers (no tensor views
-    # on the hot path); a caller-supplied buffer keeps the reference layout [B,Hq,S,Dv+1].
-    split_adapt = 0
-    if output_split is None:
-        if plan_splits:
-            # nobody looks at the partials: the library chooses the split count (with kv_split == -1 long sequences
-            # may get more than the reference's 32).  The grid has num_splits slots per sequence; a sequence uses as
-            # many as its own length asks for.
-            num_splits, split_adapt = plan_decode(q, k_cache, block_table, kv_split, k_scale=k_scale, v_scale=v_scale,
-                                                  path=path, waves_per_block=waves_per_block, max_kv_len=max_kv_len,
-                                                  v_head_dim=v_head_dim)
-        n_o = batch * q_heads * num_splits * v_head_dim
-        n_l = batch * q_heads * num_splits
-        direct = (num_splits == 1 and extra_partials is None and not fuse_combine
-                  and not (with_lse_column and lse_out is not None))
-        if no_alloc:
-            # the partials live in the library's static device array (fd_decode_noalloc); nothing is allocated here
-            if output_combine is None or fuse_combine or schedule_items:
-                raise RuntimeError("no_alloc=True needs output_combine and neither fuse_combine nor a scheduling launch")
-            if n_o + n_l > FD_NOALLOC_SCRATCH_BYTES // 4:
-                raise RuntimeError(f"no_alloc=True: {4 * (n_o + n_l)} bytes of partials exceed the library's static "
-                                   f"workspace of {FD_NOALLOC_SCRATCH_BYTES} bytes")
-            hold = None
-        elif direct:
-            # a single split: the split kernel writes the output itself, no partials and no combine launch
-            hold = None
-        elif (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
-                and workspace.is_contiguous() and workspace.numel() >= n_o + n_l):
-            # a float32 workspace that is large enough holds the partials: no allocation in the call
-            hold = workspace
-        else:
-            hold = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
-            if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
-                hold.record_stream(stream)
-        mid_ptr = hold.data_ptr() if hold is not None else None
-        lse_split_ptr = mid_ptr + 4 * n_o if hold is not None else None
-        mid_dtype = internal_partial_dtype(output_combine.dtype if output_combine is not None else q.dtype,
-                                           plan_splits, fuse_combine, n_o)
-        so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
-    else:
-        assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
-        assert output_split.shape[2] == num_splits
-        mid_ptr, lse_split_ptr, mid_dtype = output_split.data_ptr(), None, fd_dtype_of(output_split)
-        so_b, so_h, so_s = output_split.stride(0), output_split.stride(1), output_split.stride(2)
     out_cols = v_head_dim + 1 if with_lse_column else v_head_dim
     if output_combine is None:
+        if no_alloc:
+            raise RuntimeError("no_alloc=True needs output_combine")
         output_combine = torch.empty([batch, q_heads, out_cols], dtype=q.dtype, device=q.device)
+    else:
+        _require_cuda(output_combine)
     oc_st = output_combine.stride()
     assert output_combine.shape[-1] >= out_cols and oc_st[-1] == 1
-
-    if seq_order_lens is not None:
-        assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
-        assert seq_order_lens.numel() == batch
-    # Work-item order ((sequence, range) items, largest first, empty ranges last): given by the caller (the append
-    # launch computed it) or computed here by one scheduling launch.  With the caller's exact split count the items are
-    # the reference's ranges (every slot of the partial buffer is still written, empty ranges last).
-    want_items = (item_order is not None or schedule_items) and num_splits > 1 and not fuse_combine
-    if want_items and item_order is None and batch > ITEMS_UP_TO_BATCH:
-        want_items = False
-    auto_order = (AUTO_ORDER_FROM_BATCH and batch >= AUTO_ORDER_FROM_BATCH and not no_alloc
-                  and block_table.shape[1] * page_size >= 1024)
-    if (schedule_items or auto_order) and not want_items and seq_order is None and 1 < batch <= MAX_SEQ_ORDER_BATCH:
-        # per-sequence order where items do not apply -- a single split per sequence (256 ragged sequences of up to
-        # 2048 tokens: 187 us in index order, 156 us longest first), the fused combine, batches beyond the item
-        # scheduler's; still larger batches are left to the dispatcher
-        seq_order = schedule_sequences(kv_lens, stream=stream)
-        if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
-            seq_order.record_stream(stream)
-    # internal partials: splits may start on tile boundaries (the ranges are not observable)
-    p = _make_params(q, k_cache, block_table, num_splits, soft_cap, mid_dtype, fd_dtype_of(output_combine), k_scale,
-                     v_scale, path, waves_per_block, seq_order_lens, SPLIT_ALIGN if output_split is None else 0,
-                     split_adapt, 0, _hint(max_kv_len, block_table.shape[1] * page_size), v_head_dim)
-    if want_items:
-        if item_order is None:
-            item_order = item_order_buffer(batch, num_splits, q.device)
-            if stream is not None:
-                item_order.record_stream(stream)
-            check(lib.fd_schedule_items(hstream, kv_lens.data_ptr(), batch, item_order.data_ptr(), byref(p)))
-        assert item_order.dtype == torch.int32 and item_order.is_contiguous()
-        assert item_order.numel() >= 2 * batch * num_splits
-        p.seq_order_items = 1
-        p.seq_order_lens = None
-        seq_order = item_order
     ex_out = ex_lse = None
     n_extra = 0
     if extra_partials is not None:
@@ -347,15 +264,145 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert ex_lse.is_contiguous() and ex_out.dtype == output_combine.dtype
     if lse_out is not None:
         assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
-    if no_alloc:
-        if output_split is not None:
+    if seq_order_lens is not None:
+        assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
+        assert seq_order_lens.numel() == batch
+    lib = load_library()
+    hstream = stream.cuda_stream if stream is not None else stream_handle(None, q.device.index)
+    flags = ((0 if plan_splits else FD_STEP_EXACT_SPLITS) | (FD_STEP_SCHEDULE if schedule_items else 0)
+             | (0 if auto_order else FD_STEP_NO_ORDER))
+
+    if output_split is None and not fuse_combine and not no_alloc:
+        # ---- the planned step: the library chooses splits, ranges, partial type and issue order (fd_decode_planned);
+        # partials, LSEs and the order live in one workspace
+        if item_order is not None:
+            assert item_order.dtype == torch.int32 and item_order.is_contiguous()
+            seq_order = item_order
+        # (the length hint counts in steps of 1024 tokens, so that a growing batch keeps its prepared step)
+        hint = -(-max_kv_len // 1024) * 1024 if max_kv_len else 0
+        key = (q.shape, q_st, k_cache.shape, k_st, v_shape, v_st, block_table.shape[1], block_table.stride(0), oc_st,
+               q.dtype, k_cache.dtype, output_combine.dtype, kv_split, soft_cap, scale, flags, with_lse_column,
+               n_extra, path, waves_per_block, hint, k_scale is not None, item_order is not None)
+        cached = _STEP_CACHE.get(key)
+        if cached is None:
+            a = FdDecodeArgs()
+            a.stride_q_bs, a.stride_q_h = q_st[0], q_st[1]
+            a.stride_k_tok, a.stride_k_h, a.stride_v_tok, a.stride_v_h = k_st[1], k_st[2], v_st[1], v_st[2]
+            a.stride_table_bs, a.stride_obs, a.stride_oh = block_table.stride(0), oc_st[0], oc_st[1]
+            a.sm_scale, a.batch, a.num_extra, a.flags = float(scale), batch, n_extra, flags
+            a.combine_mode = FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT
+            _fill_params(a.params, q, k_cache, block_table, kv_split, soft_cap, FD_F32, fd_dtype_of(output_combine),
+                         k_scale is not None, path, waves_per_block, 0, 0, 1 if item_order is not None else 0,
+                         hint, v_head_dim)
+            need = lib.fd_workspace_bytes(byref(a.params), batch, n_extra, flags)
+            if need < 0:
+                check(int(need))
+            if len(_STEP_CACHE) > 4096:
+                _STEP_CACHE.clear()
+            cached = _STEP_CACHE[key] = (bytes(a), need)
+        image, need = cached
+        a = FdDecodeArgs.from_buffer_copy(image)
+        if (workspace is not None and isinstance(workspace, torch.Tensor) and workspace.is_cuda
+                and workspace.is_contiguous() and workspace.data_ptr() % 256 == 0
+                and workspace.numel() * workspace.element_size() >= need):
+            hold = workspace     # the caller's workspace is large enough: no allocation in the call
+        else:
+            hold = torch.empty(need, dtype=torch.uint8, device=q.device)
+            if stream is not None:   # freed on return: keep the allocator from reusing it before `stream` is done
+                hold.record_stream(stream)
+        a.q, a.k_cache, a.v_cache = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr()
+        a.workspace, a.workspace_bytes = hold.data_ptr(), need
+        a.out, a.block_table, a.kv_lens = output_combine.data_ptr(), block_table.data_ptr(), kv_lens.data_ptr()
+        if lse_out is not None:
+            a.lse_out = lse_out.data_ptr()
+        if seq_order is not None:
+            a.seq_order = seq_order.data_ptr()
+            if seq_order_lens is not None:
+                a.params.seq_order_lens = seq_order_lens.data_ptr()
+        if n_extra:
+            a.extra_out, a.extra_lse = ex_out.data_ptr(), ex_lse.data_ptr()
+        if k_scale is not None:
+            a.params.k_scale, a.params.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
+        rc = lib.fd_decode_planned(hstream, byref(a))
+        if rc:
+            check(rc)
+        return output_combine
+
+    # ---- explicit calls: the caller's own partial buffer (exactly kv_split splits with the reference's ranges, layout
+    # [B, Hq, S, Dv + 1]), the fused single launch, or partials in the library's static array.  How the step is issued
+    # still comes from the library's plan.
+    out_dtype = fd_dtype_of(output_combine)
+    lse_twice = FD_STEP_LSE_TWICE if with_lse_column and lse_out is not None else 0
+    if item_order is not None or seq_order is not None:
+        flags |= FD_STEP_NO_ORDER     # the caller brings the order
+    if output_split is not None:
+        _require_cuda(output_split)
+        assert output_split.shape[-1] == v_head_dim + 1 and output_split.stride(-1) == 1
+        num_splits = DEFAULT_KV_SPLITS if kv_split == -1 else kv_split
+        assert output_split.shape[2] == num_splits
+        if no_alloc:
             raise RuntimeError("no_alloc=True keeps the partials inside the library; output_split cannot be given")
+        plan = decode_plan(q, k_cache, block_table, num_splits, flags=flags | FD_STEP_CALLER_PARTIALS | lse_twice
+                           | (FD_STEP_FUSED if fuse_combine else 0), out_dtype=out_dtype,
+                           mid_dtype=fd_dtype_of(output_split), num_extra=n_extra, fp8=k_scale is not None, path=path,
+                           waves_per_block=waves_per_block, max_kv_len=max_kv_len, v_head_dim=v_head_dim)
+        hold = None
+        mid_ptr, lse_split_ptr = output_split.data_ptr(), None
+        so_b, so_h, so_s = output_split.stride(0), output_split.stride(1), output_split.stride(2)
+    else:
+        if no_alloc and (fuse_combine or schedule_items):
+            raise RuntimeError("no_alloc=True needs output_combine and neither fuse_combine nor a scheduling launch")
+        plan = decode_plan(q, k_cache, block_table, kv_split, flags=flags | lse_twice | (FD_STEP_NO_ORDER if no_alloc else 0)
+                           | (FD_STEP_FUSED if fuse_combine or no_alloc else 0), out_dtype=out_dtype, num_extra=n_extra,
+                           fp8=k_scale is not None, path=path, waves_per_block=waves_per_block, max_kv_len=max_kv_len,
+                           v_head_dim=v_head_dim)
+        num_splits = plan.num_splits
+        n_o = batch * q_heads * num_splits * v_head_dim
+        n_l = batch * q_heads * num_splits
+        if no_alloc:
+            # the partials live in the library's static device array (fd_decode_noalloc); nothing is allocated here
+            if n_o + n_l > FD_NOALLOC_SCRATCH_BYTES // 4:
+                raise RuntimeError(f"no_alloc=True: {4 * (n_o + n_l)} bytes of partials exceed the library's static "
+                                   f"workspace of {FD_NOALLOC_SCRATCH_BYTES} bytes")
+            hold = None
+        elif (isinstance(workspace, torch.Tensor) and workspace.dtype == torch.float32 and workspace.is_cuda
+                and workspace.is_contiguous() and workspace.numel() >= n_o + n_l):
+            hold = workspace
+        else:
+            hold = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
+            if stream is not None:
+                hold.record_stream(stream)
+        mid_ptr = hold.data_ptr() if hold is not None else None
+        lse_split_ptr = mid_ptr + 4 * n_o if hold is not None else None
+        so_b, so_h, so_s = q_heads * num_splits * v_head_dim, num_splits * v_head_dim, v_head_dim
+    want_items = (item_order is not None and num_splits > 1 and not fuse_combine) or plan.order_kind == FD_ORDER_ITEMS
+    if plan.order_kind == FD_ORDER_SEQUENCES:
+        seq_order = schedule_sequences(kv_lens, stream=stream)
+        if stream is not None:
+            seq_order.record_stream(stream)
+    p = _make_params(q, k_cache, block_table, num_splits, soft_cap, plan.mid_dtype, out_dtype, k_scale, v_scale, path,
+                     waves_per_block, seq_order_lens, plan.split_align, plan.split_adapt, 0, plan.max_kv_len, v_head_dim)
+    if want_items:
+        # (sequence, range) items, largest first, empty ranges last: given by the caller (the append launch computed
+        # it) or computed here by one scheduling launch.  With the caller's exact split count the items are the
+        # reference's ranges (every slot of the partial buffer is still written, empty ranges last).
+        if item_order is None:
+            item_order = item_order_buffer(batch, num_splits, q.device)
+            if stream is not None:
+                item_order.record_stream(stream)
+            check(lib.fd_schedule_items(hstream, kv_lens.data_ptr(), batch, item_order.data_ptr(), byref(p)))
+        assert item_order.dtype == torch.int32 and item_order.is_contiguous()
+        assert item_order.numel() >= 2 * batch * num_splits
+        p.seq_order_items = 1
+        p.seq_order_lens = None
+        seq_order = item_order
+    mode = FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT
+    if no_alloc:
         check(lib.fd_decode_noalloc(
             hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_combine.data_ptr(),
             lse_out.data_ptr() if lse_out is not None else None, float(scale), block_table.data_ptr(),
-            kv_lens.data_ptr(), batch, q_st[0], q_st[1], k_st[-3], k_st[-2], v_st[-3], v_st[-2], block_table.stride(0),
-            oc_st[0], oc_st[1], seq_order.data_ptr() if seq_order is not None else None,
-            FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
+            kv_lens.data_ptr(), batch, q_st[0], q_st[1], k_st[1], k_st[2], v_st[1], v_st[2], block_table.stride(0),
+            oc_st[0], oc_st[1], seq_order.data_ptr() if seq_order is not None else None, mode,
             ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra, byref(p)))
         return output_combine
     tickets = _tickets(q.device, hstream, batch * q_heads) if fuse_combine else None
@@ -363,16 +410,15 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), mid_ptr, lse_split_ptr,
         output_combine.data_ptr(), lse_out.data_ptr() if lse_out is not None else None, float(scale),
         block_table.data_ptr(), kv_lens.data_ptr(), batch,
-        q_st[0], q_st[1], k_st[-3], k_st[-2], v_st[-3], v_st[-2],
+        q_st[0], q_st[1], k_st[1], k_st[2], v_st[1], v_st[2],
         so_b, so_h, so_s, block_table.stride(0), oc_st[0], oc_st[1],
-        seq_order.data_ptr() if seq_order is not None else None,
-        FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT,
+        seq_order.data_ptr() if seq_order is not None else None, mode,
         ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra,
         tickets.data_ptr() if tickets is not None else None, byref(p)))
     return output_combine
 
 
-_PLAN_CACHE = {}   # fd_plan_splits results by problem shape
+_PLAN_CACHE = {}   # fd_plan_decode results by problem shape
 
 # Zero-initialised ticket counters of the fused combine, one buffer per (device, stream): calls on
 # different streams may overlap and must not share counters; the kernels leave them at zero.
@@ -393,8 +439,8 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
     """Split-KV decode + plain combine -> ``output_combine [B, Hq, Dv]`` (flash_decode.py:763-844).
 
     ``q_lens`` is accepted and ignored, as in the reference; so is ``workspace``, unless it is a
-    contiguous float32 GPU tensor of at least ``B*Hq*S*(Dv+1)`` elements, in which case the split
-    partials live in it instead of in freshly allocated memory.  Keyword ``max_kv_len=``: an upper bound of
+    contiguous GPU tensor of at least ``workspace_bytes(...)`` bytes on a 256-byte boundary, in which case partials,
+    LSEs and issue order of the step live in it instead of in freshly allocated memory.  Keyword ``max_kv_len=``: an upper bound of
     ``kv_lens`` that the caller knows on the host; the launch shape is then planned for it instead of for the block
     table's capacity (a hint only: longer sequences are still decoded in full).
     """

@@ -20,8 +20,9 @@ from typing import Optional, Tuple, Union
 import torch
 
 from .._lib import FdParams, FdQkPrep, check, fd_dtype_of, load_library, stream_handle
-from .flash_decode import (ITEMS_UP_TO_BATCH, SPLIT_ALIGN, _decode, _require_cuda, item_order_buffer,
-                           plan_decode)
+from .._lib import (FD_ORDER_ITEMS, FD_ORDER_SEQUENCES, FD_STEP_EXACT_SPLITS, FD_STEP_FUSED,
+                    FD_STEP_ORDER_FROM_APPEND)
+from .flash_decode import _decode, _require_cuda, decode_plan, item_order_buffer
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -161,9 +162,6 @@ def apply_rotary_pos_emb(x: torch.Tensor, cos_sin: torch.Tensor, position_ids: t
 
 
 _ARANGE = {}
-# Batches for which flash_attn_with_kvcache lets the append launch rank the sequences: below, every sequence's
-# workgroups start at once anyway; the upper end is what ``seq_order_out`` takes.
-SCHEDULE_MIN_BATCH, SCHEDULE_MAX_BATCH = 16, 4096
 
 
 def _dense_block_table(device, n):
@@ -228,19 +226,22 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
         if kv_lens_out is None:
             kv_lens_out = torch.empty_like(cache_seqlens)
         order = items = item_plan = None
-        if SCHEDULE_MIN_BATCH <= bsz <= SCHEDULE_MAX_BATCH and "seq_order" not in decode_kw \
-                and "item_order" not in decode_kw:
-            # the append launch also computes the decode's issue order: (sequence, range) items, largest first, when
-            # the decode cuts sequences by their own lengths and the batch fits one workgroup; else sequences, longest
-            # first
-            S, adapt = plan_decode(q[:, 0], k_cache, block_table, num_splits if num_splits > 0 else -1,
-                                   k_scale=k_scale, v_scale=v_scale, path=decode_kw.get("path", "auto"),
-                                   waves_per_block=decode_kw.get("waves_per_block", 0),
-                                   max_kv_len=decode_kw.get("max_kv_len"))
-            if S > 1 and adapt > 0 and bsz <= ITEMS_UP_TO_BATCH and not decode_kw.get("fuse_combine"):
-                items, item_plan = item_order_buffer(bsz, S, dev), (S, SPLIT_ALIGN, adapt)
+        if "seq_order" not in decode_kw and "item_order" not in decode_kw and decode_kw.get("auto_order", True):
+            # the append launch can also compute the decode's issue order, at no launch of its own: the library's
+            # plan says whether that pays for this batch and which kind -- (sequence, range) items, largest first, or
+            # sequences, longest first
+            plan = decode_plan(q[:, 0], k_cache, block_table, num_splits if num_splits > 0 else -1,
+                               flags=FD_STEP_ORDER_FROM_APPEND
+                               | (0 if decode_kw.get("plan_splits", True) else FD_STEP_EXACT_SPLITS)
+                               | (FD_STEP_FUSED if decode_kw.get("fuse_combine") else 0),
+                               out_dtype=fd_dtype_of(q), fp8=k_scale is not None, path=decode_kw.get("path", "auto"),
+                               waves_per_block=decode_kw.get("waves_per_block", 0),
+                               max_kv_len=decode_kw.get("max_kv_len"), v_head_dim=v_cache.shape[-1])
+            if plan.order_kind == FD_ORDER_ITEMS:
+                items = item_order_buffer(bsz, plan.num_splits, dev)
+                item_plan = (plan.num_splits, plan.split_align, plan.split_adapt)
                 decode_kw["item_order"] = items
-            else:
+            elif plan.order_kind == FD_ORDER_SEQUENCES:
                 order = torch.empty((2, bsz), dtype=torch.int32, device=dev)
                 decode_kw["seq_order"], decode_kw["seq_order_lens"] = order[0], order[1]
         prep_q = cos_sin_cache is not None or q_norm is not None
