@@ -358,7 +358,10 @@ FD_API int fd_decode_planned(void* stream, const fd_decode_args* args);
  *   - every GPU the library is used on holds its own copy of the array until the process ends;
  *   - all calls on one GPU share that array: calls that may overlap on one GPU (different streams, graphs
  *     replayed concurrently) race on it -- serialise them, or use fd_decode with workspaces of your own;
- *     the array keeps the last call's partials, which the next call overwrites before it reads them.
+ *     the array keeps the last call's partials, which the next call overwrites before it reads them;
+ *   - the first call on a device looks up the array's device address (hipGetSymbolAddress, once per device): make
+ *     that call outside a stream capture -- one eager step before the graph is recorded -- since a symbol lookup is
+ *     module set-up and not a capturable operation; every later call only launches kernels.
  */
 #define FD_NOALLOC_SCRATCH_BYTES (16u << 20)
 FD_API int fd_decode_noalloc(void* stream, const void* q, const void* k_cache, const void* v_cache,

@@ -1,6 +1,6 @@
 /*
  * A consumer of the C ABI with no Python in the loop: fills a small paged decode problem, runs fd_decode (and
- * fd_decode_noalloc, fd_schedule, fd_plan_splits, fd_kv_append) from libflash_decode_gfx950.so on the GPU and checks the result
+ * fd_decode_planned, fd_decode_noalloc, fd_schedule, fd_plan_splits, fd_kv_append) from libflash_decode_gfx950.so on the GPU and checks the result
  * against the plain-C oracle (oracle/c/ref_decode.c).  Exit code 0 = all checks passed.
  *
  *   gcc -O2 -std=c11 -D__HIP_PLATFORM_AMD__ tests/c_abi/run_c_abi.c oracle/c/ref_decode.c -Iinclude -I/opt/rocm/include \
@@ -116,6 +116,54 @@ int main(void) {
     if (!(fabs((double)lse[i] - (double)ref_lse[i]) <= 1e-5 * fmax(1.0, fabs((double)ref_lse[i])))) ++bad;
   }
   printf("fd_decode (fp32, soft cap, scheduled, %d planned of %d splits): max |out - ref| = %.3e\n", planned, S, worst);
+
+  /* the planned step: the library picks splits, ranges, partial type and issue order; the caller only brings a
+     workspace of the size the library names -- the path a binding should take when nobody looks at the partials */
+  {
+    fd_decode_args a;
+    memset(&a, 0, sizeof(a));
+    a.params = p;
+    a.params.num_splits = -1;   /* no hint */
+    fd_launch_plan lp;
+    FD_OK_OR_DIE(fd_plan_decode(&a.params, B, 0, FD_STEP_SCHEDULE, &lp));
+    const int64_t need = fd_workspace_bytes(&a.params, B, 0, FD_STEP_SCHEDULE);
+    if (need <= 0 || need != lp.workspace_bytes || lp.num_splits < 1 || lp.order_kind == FD_ORDER_NONE) {
+      fprintf(stderr, "fd_workspace_bytes -> %lld (plan %lld, %d splits, order %d)\n", (long long)need,
+              (long long)lp.workspace_bytes, lp.num_splits, lp.order_kind);
+      return 1;
+    }
+    void *dws = NULL, *dout3 = NULL, *dlse3 = NULL;
+    HIP_OK(hipMalloc(&dws, (size_t)need));
+    HIP_OK(hipMalloc(&dout3, nq * 4));
+    HIP_OK(hipMalloc(&dlse3, sizeof(ref_lse)));
+    HIP_OK(hipMemset(dws, 0xff, (size_t)need));   /* the workspace's contents mean nothing: NaNs */
+    a.q = dq; a.k_cache = dk; a.v_cache = dv; a.workspace = dws; a.workspace_bytes = need; a.out = dout3;
+    a.lse_out = (float*)dlse3; a.block_table = (const int32_t*)dbt; a.kv_lens = (const int32_t*)dlens;
+    a.stride_q_bs = (int64_t)HQ * D; a.stride_q_h = D; a.stride_k_tok = (int64_t)HKV * D; a.stride_k_h = D;
+    a.stride_v_tok = (int64_t)HKV * D; a.stride_v_h = D; a.stride_table_bs = MAXP; a.stride_obs = (int64_t)HQ * D;
+    a.stride_oh = D; a.sm_scale = scale; a.batch = B; a.combine_mode = FD_COMBINE_SPLIT; a.flags = FD_STEP_SCHEDULE;
+    FD_OK_OR_DIE(fd_decode_planned(NULL, &a));
+    HIP_OK(hipDeviceSynchronize());
+    float* out3 = (float*)malloc(nq * 4);
+    float lse3[B * HQ];
+    HIP_OK(hipMemcpy(out3, dout3, nq * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(lse3, dlse3, sizeof(lse3), hipMemcpyDeviceToHost));
+    double worst3 = 0.0;
+    for (size_t i = 0; i < nq; ++i) {
+      const double e = fabs((double)out3[i] - (double)ref_out[i]);
+      if (e > worst3) worst3 = e;
+      if (!(e <= 2e-4)) ++bad;
+    }
+    for (int i = 0; i < B * HQ; ++i) {
+      if (isinf(ref_lse[i])) { if (!(isinf(lse3[i]) && lse3[i] < 0)) ++bad; continue; }
+      if (!(fabs((double)lse3[i] - (double)ref_lse[i]) <= 1e-5 * fmax(1.0, fabs((double)ref_lse[i])))) ++bad;
+    }
+    printf("fd_decode_planned (%d splits, workspace %lld bytes, order kind %d): max |out - ref| = %.3e\n", lp.num_splits,
+           (long long)need, lp.order_kind, worst3);
+    /* a workspace that is too small is refused with the size in the message, nothing is launched */
+    a.workspace_bytes = need - 1;
+    if (fd_decode_planned(NULL, &a) != FD_ERR_INVALID_ARG || strstr(fd_last_error(), "workspace") == NULL) ++bad;
+  }
 
   /* the entry point that allocates nothing (partials in the library's static device array): the same bits */
   void *dout2 = NULL, *dlse2 = NULL;

@@ -1,5 +1,5 @@
 """Runs the C consumer of the ABI (tests/c_abi/run_c_abi.c: no Python between the caller and the library) on the GPU;
-it checks fd_decode / fd_schedule / fd_plan_splits / fd_kv_append against the plain-C oracle and exits 0 on success."""
+it checks fd_decode / fd_decode_planned / fd_schedule / fd_plan_splits / fd_kv_append against the plain-C oracle and exits 0 on success."""
 import importlib.util
 import os
 import subprocess

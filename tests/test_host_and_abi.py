@@ -259,3 +259,150 @@ def test_a_stale_library_is_rebuilt_not_silently_used(fd, monkeypatch):
     assert calls == [True]
     monkeypatch.setenv("FD_LIBRARY_PATH", "/somewhere/else.so")            # an explicit library is the caller's business
     assert b.ensure_built() == "/somewhere/else.so"
+
+
+def _struct_fields(name):
+    """(ctype, is_pointer, field, array length) of the members of a struct in the header, in order."""
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), _header_text(), re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    out = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        m = re.match(r"(?:const\s+)?(\w+)\s*(\*?)\s*(.*)$", decl, re.S)
+        ctype, ptr, names = m.group(1), m.group(2), m.group(3)
+        for n in names.split(","):
+            n = n.strip()
+            star = ptr or ("*" if n.startswith("*") else "")
+            n = n.lstrip("* ")
+            arr = re.match(r"(\w+)\[(\d+)\]", n)
+            out.append((ctype, bool(star), arr.group(1) if arr else n, int(arr.group(2)) if arr else 0))
+    return out
+
+
+def test_plan_and_step_structs_mirror_the_header(fd):
+    L = fd._lib
+    simple = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "float": ctypes.c_float, "fd_params": L.FdParams}
+    for cname, mirror in (("fd_launch_plan", L.FdLaunchPlan), ("fd_decode_args", L.FdDecodeArgs)):
+        fields = _struct_fields(cname)
+        assert [f[2] for f in fields] == [n for n, _ in mirror._fields_], cname
+        for (ctype, ptr, name, arr), (_, pytype) in zip(fields, mirror._fields_):
+            expect = ctypes.c_void_p if ptr else simple[ctype]
+            if arr:
+                expect = expect * arr
+            assert pytype is expect or (arr and pytype._type_ is expect._type_ and pytype._length_ == arr), (cname, name)
+    enums = dict(re.findall(r"\b(FD_[A-Z0-9_]+)\s*=\s*(-?\d+)", _header_text()))
+    for name in ("FD_STEP_EXACT_SPLITS", "FD_STEP_SCHEDULE", "FD_STEP_NO_ORDER", "FD_STEP_FUSED", "FD_STEP_LSE_TWICE",
+                 "FD_STEP_CALLER_PARTIALS", "FD_STEP_ORDER_FROM_APPEND", "FD_ORDER_NONE", "FD_ORDER_SEQUENCES",
+                 "FD_ORDER_ITEMS"):
+        assert int(enums[name]) == getattr(L, name), name
+    # the stand-alone binding repeats fd_decode_args
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(
+        "fd_reference_binding_cpu2", os.path.join(ROOT, "triton-distributed_amd", "reference_binding.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert [(n, t) for n, t in mod.FdDecodeArgs._fields_[:-1]] == [(n, t) for n, t in L.FdDecodeArgs._fields_[:-1]]
+    assert ctypes.sizeof(mod.FdDecodeArgs) == ctypes.sizeof(L.FdDecodeArgs)
+
+
+def _plan(fd, B, Hq, Hkv, S, max_pages, P=16, kv=None, D=128, flags=0, out=None, extra=0, mid=0, max_kv_len=0):
+    L = fd._lib
+    lib = fd.load_library()
+    kv = L.FD_BF16 if kv is None else kv
+    out = L.FD_BF16 if out is None else out
+    p = L.FdParams()
+    p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits = Hq, Hkv, D, P, S
+    p.num_pages, p.max_pages_per_seq, p.q_dtype, p.kv_dtype, p.out_dtype, p.mid_dtype = max_pages * B, max_pages, out, kv, out, mid
+    p.max_kv_len = max_kv_len
+    lp = L.FdLaunchPlan()
+    rc = lib.fd_plan_decode(ctypes.byref(p), B, extra, flags, ctypes.byref(lp))
+    assert rc == 0, lib.fd_last_error()
+    assert lib.fd_workspace_bytes(ctypes.byref(p), B, extra, flags) == lp.workspace_bytes
+    return lp
+
+
+def test_launch_plan_of_the_five_configs_and_the_published_sweep(fd):
+    """fd_plan_decode pins the whole launch shape -- splits, ranges, partial type, order kind, waves, members, chunk,
+    grid -- for the benchmark configurations and for the shapes of the reference's published sweep (one query,
+    96 / 12 heads, fp16, page size 1, test_decode_attn.py:303-312)."""
+    L = fd._lib
+    F32, F16, BF16, FP8 = L.FD_F32, L.FD_F16, L.FD_BF16, L.FD_FP8_E4M3
+
+    def shape(lp):
+        return (lp.num_splits, lp.split_adapt, lp.split_align, lp.mid_dtype, lp.direct, lp.order_kind, lp.mfma, lp.tile,
+                lp.waves_per_head, lp.members, lp.chunk, tuple(lp.grid))
+
+    # config 2: planned, exactly 32 splits (chunked work items, 16-bit partials), caller-visible fp32 / bf16 partials
+    assert shape(_plan(fd, 8, 32, 8, 32, 512)) == (8, 8, 64, F32, 0, 0, 1, 32, 2, 2, 1, (4, 8, 8))
+    assert shape(_plan(fd, 8, 32, 8, 32, 512, flags=L.FD_STEP_EXACT_SPLITS)) == (32, 0, 64, BF16, 0, 0, 1, 32, 2, 2, 4, (4, 8, 8))
+    for mid in (F32, BF16):
+        lp = _plan(fd, 8, 32, 8, 32, 512, flags=L.FD_STEP_CALLER_PARTIALS, mid=mid)
+        assert shape(lp) == (32, 0, 0, mid, 0, 0, 1, 32, 2, 2, 4, (4, 8, 8)) and lp.workspace_bytes == 0
+    # config 3: one sequence of 131072 tokens + 7 extra partials
+    assert shape(_plan(fd, 1, 32, 8, 32, 8192, extra=7)) == (64, 64, 64, F32, 0, 0, 1, 32, 2, 2, 1, (4, 1, 64))
+    # config 4: ragged batch of 64 -- the plain step ranks its sequences, the scheduled one its (sequence, range) items
+    lp = _plan(fd, 64, 32, 8, 32, 2048)
+    assert shape(lp) == (8, 1, 64, BF16, 0, L.FD_ORDER_SEQUENCES, 1, 32, 2, 2, 1, (4, 64, 8)) and lp.order_bytes == 256
+    lp = _plan(fd, 64, 32, 8, 32, 2048, flags=L.FD_STEP_SCHEDULE)
+    assert shape(lp) == (8, 1, 64, BF16, 0, L.FD_ORDER_ITEMS, 1, 32, 2, 2, 1, (4, 8, 64)) and lp.order_bytes == 2 * 64 * 8 * 4
+    assert _plan(fd, 64, 32, 8, 32, 2048, flags=L.FD_STEP_NO_ORDER).order_kind == L.FD_ORDER_NONE
+    # config 5: fp8 cache, four sibling KV heads per workgroup; exactly 64 splits: written-through 16-bit partials
+    assert shape(_plan(fd, 32, 64, 8, 64, 1024, kv=FP8)) == (4, 4, 64, BF16, 0, 0, 1, 64, 2, 4, 1, (2, 32, 4))
+    lp = _plan(fd, 32, 64, 8, 64, 1024, kv=FP8, flags=L.FD_STEP_EXACT_SPLITS)
+    assert shape(lp) == (64, 0, 64, BF16, 0, 0, 1, 64, 1, 4, 4, (2, 16, 32)) and lp.store_through == 1
+    # config 1: fp32 plumbing on the VALU kernel
+    lp = _plan(fd, 1, 8, 2, 4, 1, P=1024, kv=F32, out=F32)
+    assert (lp.mfma, lp.mid_dtype, lp.num_splits, lp.waves_per_head) == (0, F32, 32, 8)
+    # the published sweep: the library's own split count
+    for tokens, expect in ((8192, (21, 32, 4, 1, (12, 1, 21))), (16384, (21, 32, 4, 1, (12, 1, 21))),
+                           (32768, (42, 64, 2, 2, (6, 1, 42))), (65536, (42, 64, 2, 2, (6, 1, 42))),
+                           (131072, (42, 64, 2, 2, (6, 1, 42))), (1048576, (42, 64, 2, 2, (6, 1, 42)))):
+        lp = _plan(fd, 1, 96, 12, -1, tokens, P=1, kv=F16, out=F16)
+        assert (lp.num_splits, lp.split_adapt, lp.waves_per_head, lp.members, tuple(lp.grid)) == expect, tokens
+        assert (lp.mid_dtype, lp.order_kind, lp.direct, lp.chunk, lp.tile) == (F32, 0, 0, 1, 32)
+    # a large batch of short sequences: one split, written straight to the output
+    lp = _plan(fd, 64, 32, 8, 32, 128)
+    assert (lp.num_splits, lp.direct, lp.partial_bytes > 0) == (1, 1, True)
+    assert _plan(fd, 64, 32, 8, 32, 128, flags=L.FD_STEP_LSE_TWICE).direct == 0
+    assert _plan(fd, 64, 32, 8, 32, 128, extra=1).direct == 0
+    # the host-side length hint replaces the capacity, in steps of 1024 tokens
+    wide = _plan(fd, 64, 32, 8, 32, 8192, max_kv_len=1000)
+    assert (wide.max_kv_len, wide.num_splits) == (1024, 1) and _plan(fd, 64, 32, 8, 32, 8192).num_splits == 32
+    # an order that costs no launch pays from 16 sequences on
+    assert _plan(fd, 16, 32, 8, 32, 2048, flags=L.FD_STEP_ORDER_FROM_APPEND).order_kind == L.FD_ORDER_ITEMS
+    assert _plan(fd, 15, 32, 8, 32, 2048, flags=L.FD_STEP_ORDER_FROM_APPEND).order_kind == L.FD_ORDER_NONE
+    assert _plan(fd, 256, 32, 8, 32, 2048, flags=L.FD_STEP_SCHEDULE).order_kind == L.FD_ORDER_SEQUENCES
+    assert _plan(fd, 5000, 32, 8, 32, 64, flags=L.FD_STEP_SCHEDULE).order_kind == L.FD_ORDER_NONE
+
+
+def test_decode_planned_validates_before_it_launches(fd):
+    L = fd._lib
+    lib = fd.load_library()
+    assert lib.fd_decode_planned(None, None) == -1
+    a = L.FdDecodeArgs()
+    a.batch = 2
+    fake = 0x10000
+    a.q = a.k_cache = a.v_cache = a.out = a.block_table = a.kv_lens = fake
+    p = a.params
+    p.q_heads, p.kv_heads, p.head_dim, p.page_size, p.num_splits, p.num_pages, p.max_pages_per_seq = 32, 8, 128, 16, 32, 64, 32
+    p.q_dtype = p.kv_dtype = p.out_dtype = L.FD_BF16
+    a.flags = 1 << 10
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1 and b"flags" in lib.fd_last_error()
+    a.flags, a.combine_mode = 0, L.FD_COMBINE_RANK
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1 and b"combine_mode" in lib.fd_last_error()
+    a.combine_mode = L.FD_COMBINE_SPLIT
+    need = lib.fd_workspace_bytes(ctypes.byref(p), 2, 0, 0)
+    assert need > 0
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1 and str(need).encode() in lib.fd_last_error()   # no workspace
+    a.workspace, a.workspace_bytes = fake + 16, need
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1 and b"aligned" in lib.fd_last_error()
+    a.workspace, a.workspace_bytes = fake, need - 1
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1 and b"workspace" in lib.fd_last_error()
+    p.q_heads = 30
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == -1
+    assert lib.fd_workspace_bytes(ctypes.byref(p), 2, 0, 0) == -1
+    assert lib.fd_plan_decode(ctypes.byref(p), 2, 0, 0, None) == -1
+    a.batch = 0
+    assert lib.fd_decode_planned(None, ctypes.byref(a)) == 0   # an empty batch is a no-op

@@ -12,6 +12,9 @@ from helpers import DEV, assert_lse_close, assert_out_close, oracle_decode
 pytestmark = pytest.mark.gpu
 
 
+_WARM = {}
+
+
 def _params(fd, g, num_splits, out, split_adapt=0, split_align=0):
     L = fd._lib
     p = L.FdParams()
@@ -47,12 +50,16 @@ def _both(fd, wl, num_splits, mode=0, split_adapt=0, split_align=0):
     lse_arg_b = None if mode == L.FD_COMBINE_SPLIT_LSE else lse_b.data_ptr()
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(DEV)[0]
     L.check(lib.fd_decode_noalloc(
         stream, g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), out_a.data_ptr(), lse_arg_a,
         float(g.scale), g.block_table.data_ptr(), g.kv_lens.data_ptr(), B, g.q.stride(0), g.q.stride(1),
         g.k_cache.stride(-3), g.k_cache.stride(-2), g.v_cache.stride(-3), g.v_cache.stride(-2),
         g.block_table.stride(0), out_a.stride(0), out_a.stride(1), None, mode, None, None, 0, byref(p)))
     assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before   # torch's allocator was not touched
+    if _WARM.get("done"):   # (the very first call on a device looks up the static array's address: module set-up)
+        assert torch.cuda.mem_get_info(DEV)[0] == free_before                   # ... and neither was the driver's
+    _WARM["done"] = True
     n_o = B * Hq * num_splits * D
     L.check(lib.fd_decode(
         stream, g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), mid.data_ptr(),
@@ -120,3 +127,108 @@ def test_no_alloc_rejects_what_does_not_fit(fd):
     assert b"static workspace" in lib.fd_last_error()
     torch.cuda.synchronize()
     assert not out.any()   # nothing was launched
+
+
+def test_no_alloc_keyword_of_the_python_wrappers(fd):
+    """``no_alloc=True``: the wrappers plan the step as usual and keep the partials in the library's static array."""
+    cases = [
+        fd.utils.make_paged_workload("noalloc_kw_bf16", [1320, 2049, 463, 18], 32, 8, 128, 16, torch.bfloat16, 32, seed=51),
+        fd.utils.make_paged_workload("noalloc_kw_fp8", [777, 33, 5000], 64, 8, 128, 16, torch.bfloat16, 32, seed=52,
+                                     fp8_kv=True),
+        fd.utils.make_paged_workload("noalloc_kw_d256", [300, 1, 900], 16, 8, 256, 1, torch.float16, 32, seed=53),
+        fd.utils.make_paged_workload("noalloc_kw_direct", [200] * 70, 32, 8, 128, 16, torch.bfloat16, 32, seed=54),
+    ]
+    for wl in cases:
+        g = wl.to(DEV)
+        B, Hq, D = g.q.shape
+        kw = dict(k_scale=g.k_scale, v_scale=g.v_scale) if g.k_scale is not None else {}
+        ref, ref_lse = oracle_decode(wl)
+        # plain wrapper with a separate fp32 LSE
+        out = torch.zeros(B, Hq, D, dtype=g.q.dtype, device=DEV)
+        lse = torch.zeros(B, Hq, dtype=torch.float32, device=DEV)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+        same = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, [1] * B, g.kv_lens, g.block_table, g.scale,
+                                       output_combine=out, kv_split=g.kv_split, lse_out=lse, no_alloc=True, **kw)
+        assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
+        torch.cuda.synchronize()
+        assert same is out
+        assert_out_close(out.cpu(), ref)
+        assert_lse_close(lse.cpu(), ref_lse)
+        # bit-identical to the same step with the partials in freshly allocated memory
+        usual = fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, [1] * B, g.kv_lens, g.block_table, g.scale,
+                                        kv_split=g.kv_split, auto_order=False, **kw)
+        torch.cuda.synchronize()
+        if fd.kernels.flash_decode.decode_plan(g.q, g.k_cache, g.block_table, g.kv_split, fp8=g.k_scale is not None
+                                               ).mid_dtype == fd._lib.FD_F32:
+            assert torch.equal(out.cpu().view(torch.int16), usual.cpu().view(torch.int16)), wl.name
+        # intra-rank wrapper: merged LSE in the output's last column
+        out1 = torch.zeros(B, Hq, D + 1, dtype=g.q.dtype, device=DEV)
+        fd.gqa_fwd_batch_decode_intra_rank(g.q, g.k_cache, g.v_cache, None, [1] * B, g.kv_lens, g.block_table, g.scale,
+                                           output_combine=out1, kv_split=g.kv_split, no_alloc=True, **kw)
+        torch.cuda.synchronize()
+        assert_out_close(out1[..., :D].cpu(), ref)
+        assert_lse_close(out1[..., D].float().cpu(), ref_lse, rtol=1e-2)   # the column has the output's 16-bit type
+    with pytest.raises(RuntimeError, match="output_combine"):
+        g = cases[0].to(DEV)
+        fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale, no_alloc=True)
+    with pytest.raises(RuntimeError, match="output_split"):
+        fd.gqa_fwd_batch_decode(g.q, g.k_cache, g.v_cache, None, None, g.kv_lens, g.block_table, g.scale, no_alloc=True,
+                                output_combine=torch.empty(4, 32, 128, dtype=torch.bfloat16, device=DEV),
+                                output_split=torch.empty(4, 32, 32, 129, dtype=torch.float32, device=DEV))
+
+
+def test_no_alloc_step_in_a_hip_graph(fd):
+    """What the entry point is for: a decode step captured into a HIP graph (no allocation may happen under capture)
+    and replayed with other lengths.  One eager call on the device comes first -- it looks up the static array's
+    address, which is module set-up and not for a capture -- and every replay is checked against the eager result,
+    with the program's own eager work and synchronisations between the replays."""
+    L = fd._lib
+    lib = fd.load_library()
+    wl = fd.utils.make_paged_workload("noalloc_graph", [1320, 2049, 463], 32, 8, 128, 16, torch.bfloat16, 32, seed=61)
+    g = wl.to(DEV)
+    B, Hq, D = g.q.shape
+    S = 8
+    out = torch.zeros(B, Hq, D, dtype=g.q.dtype, device=DEV)
+    lse = torch.zeros(B, Hq, dtype=torch.float32, device=DEV)
+    lens = g.kv_lens.clone()
+    p = _params(fd, g, S, out, split_adapt=2, split_align=64)
+
+    def launch(stream):
+        L.check(lib.fd_decode_noalloc(
+            stream, g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            float(g.scale), g.block_table.data_ptr(), lens.data_ptr(), B, g.q.stride(0), g.q.stride(1),
+            g.k_cache.stride(-3), g.k_cache.stride(-2), g.v_cache.stride(-3), g.v_cache.stride(-2),
+            g.block_table.stride(0), out.stride(0), out.stride(1), None, 0, None, None, 0, byref(p)))
+
+    def eager(new_lens):
+        lens.copy_(torch.tensor(new_lens, dtype=torch.int32))
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        res = out.clone(), lse.clone()
+        out.zero_()
+        lse.zero_()
+        return res
+
+    eager(wl.kv_lens.tolist())   # the first call on the device, outside any capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for new_lens in ([1320, 2049, 463], [70, 0, 2049], [2049, 2049, 2049], [1, 17, 33], [1320, 2049, 463]):
+        want_out, want_lse = eager(new_lens)          # eager work between the replays
+        lens.copy_(torch.tensor(new_lens, dtype=torch.int32))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), want_out.view(torch.int16)), new_lens
+        assert torch.equal(lse.view(torch.int32), want_lse.view(torch.int32)), new_lens
+        w2 = fd.utils.make_paged_workload("noalloc_graph", [1320, 2049, 463], 32, 8, 128, 16, torch.bfloat16, 32, seed=61)
+        w2.kv_lens = torch.tensor(new_lens, dtype=torch.int32)
+        ref, ref_lse = oracle_decode(w2)
+        assert_out_close(out.cpu(), ref)
+        assert_lse_close(lse.cpu(), ref_lse)
+        out.zero_()
+        lse.zero_()

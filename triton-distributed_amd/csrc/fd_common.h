@@ -201,12 +201,14 @@ __device__ __forceinline__ u32x2 load_stream_b64(const void* p) { return __built
 // Four consecutive values of a partial row that starts on a multiple of four elements (SplitArgs::vec_out): one
 // 128-bit store for fp32, one 64-bit store of four packed values for fp16 / bf16.  through: written through to memory
 // (sc0 sc1).  The write-through form is inline assembly, which the compiler does not count in vmcnt: only for stores
-// that no vector-memory load of the same wave follows.
+// that no vector-memory load of the same wave follows.  Nor does the compiler's hazard pass look inside it: a store of
+// more than 64 bits needs wait states before a VALU instruction may overwrite its data registers, so the 128-bit
+// forms carry their own s_nop.
 __device__ __forceinline__ void store_partial4(void* base, int64_t off, int dtype, f32x4 o, bool through) {
   if (dtype == FD_F32) {
     float* p = (float*)base + off;
     if (through) {
-      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(o) : "memory");
+      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(o) : "memory");
     } else {
       *(f32x4*)p = o;
     }
@@ -816,7 +818,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
       const f32x4 v = *(const f32x4*)((const float*)rows + h * D + d);
       float* p = (float*)a.out + off;
       if (through) {
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
       } else {
         *(f32x4*)p = v;
       }
