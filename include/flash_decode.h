@@ -74,6 +74,25 @@ typedef enum fd_combine_mode {
  * flash_decode.py:103-109) plus what a typed C ABI needs to know about the
  * buffers.  Zero-initialise, then fill.
  */
+/*
+ * Sequence-parallel decode on one rank (SpGQAFlashDecodeAttention.forward,
+ * python/triton_dist/layers/nvidia/sp_flash_decode_layer.py:83-185): the reference runs the local decode with the
+ * intra-rank combine (:107-110), copies the result into this rank's slot of a staged buffer [R, B, Hq, Dv + 1]
+ * (:136-138), allgathers the other slots (:139) and launches the inter-rank combine over all of them (:173-183).
+ * With this block in fd_params the combine of fd_decode / fd_decode_planned / fd_combine (split modes) does the last
+ * three steps in its one launch: it merges the local split partials, writes that merge into `local_out` -- the slot a
+ * push to the other ranks would be sent from -- and merges it with the extra partials, which then stand for the other
+ * ranks in rank order (this rank left out), each counting for sequence b iff its rank holds tokens of it
+ * (flash_decode.py:513-515).
+ */
+typedef struct fd_rank_merge {
+  const int32_t* rank_lens; /* global_kv_lens [num_extra + 1, batch] int32 (device): every rank's local kv length     */
+  int32_t this_rank;        /* the row of rank_lens that is this rank's own; extra e is rank e < this_rank ? e : e + 1 */
+  int32_t local_dtype;      /* fd_dtype of local_out                                                                  */
+  void* local_out;          /* NULL, or [batch, Hq, Dv + 1]: merge of the local split partials, LSE at column Dv       */
+  int64_t stride_lb, stride_lh; /* element strides of local_out                                                        */
+} fd_rank_merge;
+
 typedef struct fd_params {
   int32_t q_heads;          /* Hq                                                  */
   int32_t kv_heads;         /* Hkv; Hq % Hkv == 0                                  */
@@ -128,6 +147,8 @@ typedef struct fd_params {
                                to 16 query heads per KV head runs on the MFMA kernel, everything else on
                                the VALU kernel (FD_ERR_UNSUPPORTED for the other shapes with
                                FD_PATH_MFMA, with an fp8 cache and in fd_kv_append).            */
+  const fd_rank_merge* rank_merge; /* NULL, or how the extra partials of this step stand for other ranks (above);
+                               not with a ticket buffer (the fused combine)                                   */
 } fd_params;
 
 /*

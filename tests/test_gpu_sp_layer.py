@@ -71,18 +71,30 @@ def test_sp_layer_matches_oracle_on_concatenated_cache(fd, R, Hq, Hkv, P, dtype)
         fd.gqa_fwd_batch_decode_intra_rank(gq, ks[r].to(DEV), vs[r].to(DEV), None, [1] * B, glens[r].contiguous(),
                                            bts[r].to(DEV), scale, output_combine=oc, kv_split=32)
         parts.append(oc)
-    for rank in (0, R - 1):
+    # both forms of the forward: the other ranks' partials merged where they are (two launches), and the reference's
+    # steps one by one through the staged slots
+    for rank, staged in ((0, False), (R - 1, False), (0, True), (R - 1, True)):
         layer = fd.SpGQAFlashDecodeAttention(rank, 0, R, 1, Hq, Hkv, D, D, page_size=P, scale=scale, soft_cap=0,
-                                             max_allowed_batch=B, stages=3)
+                                             max_allowed_batch=B, stages=3, staged_exchange=staged)
         others = [r for r in range(R) if r != rank]
         r_out = torch.stack([parts[r][..., :D] for r in others]).to(dtype)
         r_lse = torch.stack([parts[r][..., D] for r in others]).contiguous()
+        if rank != 1:
+            # rank 1 holds nothing of sequence 1: what it sends for that sequence must not be looked at
+            r_out[others.index(1), 1] = float("nan")
+            r_lse[others.index(1), 1] = float("nan")
         for _ in range(4):                                # the staging ring rotates
             out = layer(gq, ks[rank].to(DEV), vs[rank].to(DEV), glens, bts[rank].to(DEV),
                         remote_partials=(r_out, r_lse))
         torch.cuda.synchronize()
         torch.testing.assert_close(out.float().cpu(), ref, atol=0.05, rtol=1e-2)
         assert_out_close(out, ref)
+        # this rank's slot of the staged buffer holds its own merged partial (out, lse): what a push would send
+        stage = layer.ag_buffer[(layer.signal_target - 1) % layer.stages][:R * B * Hq * (D + 1) * 4]
+        slot = stage.view(torch.float32).view(R, B, Hq, D + 1)[rank].cpu()
+        mine = parts[rank].cpu()
+        assert_out_close(slot[..., :D], mine[..., :D], atol=1e-5, rel=False)
+        assert_lse_close(slot[..., D], mine[..., D], rtol=1e-6)
         layer.finalize()
 
 

@@ -33,13 +33,13 @@ def test_enums_and_params_struct_mirror_the_header(fd):
     for name in ("FD_F32", "FD_F16", "FD_BF16", "FD_FP8_E4M3", "FD_PATH_AUTO", "FD_PATH_VALU", "FD_PATH_MFMA",
                  "FD_COMBINE_SPLIT", "FD_COMBINE_SPLIT_LSE", "FD_COMBINE_RANK"):
         assert int(enums[name]) == getattr(L, name), name
-    body = re.search(r"typedef struct fd_params \{(.*?)\} fd_params;", text, re.S).group(1)
-    fields = re.findall(r"^\s*(?:const\s+)?(int32_t|float)\s*(\*?)\s*(\w+);", body, re.M)
-    mirror = [(n, t) for n, t in L.FdParams._fields_]
-    assert [f[2] for f in fields] == [n for n, _ in mirror]
-    for (ctype, ptr, name), (_, pytype) in zip(fields, mirror):
-        expect = ctypes.c_void_p if ptr else (ctypes.c_int32 if ctype == "int32_t" else ctypes.c_float)
-        assert pytype is expect, name
+    simple = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "float": ctypes.c_float}
+    for cname, struct in (("fd_params", L.FdParams), ("fd_rank_merge", L.FdRankMerge), ("fd_qk_prep", L.FdQkPrep)):
+        fields = _struct_fields(cname)
+        mirror = [(n, t) for n, t in struct._fields_]
+        assert [f[2] for f in fields] == [n for n, _ in mirror], cname
+        for (ctype, ptr, name, _), (_, pytype) in zip(fields, mirror):
+            assert pytype is (ctypes.c_void_p if ptr else simple[ctype]), (cname, name)
 
 
 def test_stand_alone_reference_binding_mirrors_the_same_structs(fd):

@@ -62,6 +62,15 @@ class FdParams(Structure):
         ("max_kv_len", c_int32),
         ("seq_order_items", c_int32),
         ("v_head_dim", c_int32),
+        ("rank_merge", c_void_p),
+    ]
+
+
+class FdRankMerge(Structure):
+    """Mirror of ``struct fd_rank_merge``."""
+    _fields_ = [
+        ("rank_lens", c_void_p), ("this_rank", c_int32), ("local_dtype", c_int32), ("local_out", c_void_p),
+        ("stride_lb", c_int64), ("stride_lh", c_int64),
     ]
 
 

@@ -573,6 +573,8 @@ int fd_decode(void* stream, const void* q, const void* k_cache, const void* v_ca
     return fail(FD_ERR_INVALID_ARG, "fd_decode: num_extra %d needs extra_out and extra_lse", num_extra);
   if (p && (!dtype_size(p->out_dtype) || p->out_dtype == FD_FP8_E4M3))
     return fail(FD_ERR_UNSUPPORTED, "fd_decode: out_dtype %d", p->out_dtype);
+  if (p && p->rank_merge && tickets)
+    return fail(FD_ERR_INVALID_ARG, "fd_decode: rank_merge is not available with a ticket buffer (fused combine)");
   if (!out_split) {
     // One split and nothing else to merge: its normalised partial IS the result.  The split kernel writes
     // it (and the LSE) in the output's place and dtype; no combine launch.
@@ -780,6 +782,24 @@ static int combine_impl(void* stream, const void* mid_o, const float* mid_lse, v
   if (p->max_pages_per_seq > 0 && p->page_size > 0) {
     const int64_t cap = (int64_t)p->max_pages_per_seq * p->page_size;
     if (cap < a.capacity) a.capacity = cap;
+  }
+  if (const fd_rank_merge* rm = p->rank_merge) {
+    if (mode == FD_COMBINE_RANK) return fail(FD_ERR_INVALID_ARG, "fd_combine: rank_merge goes with the split modes");
+    if (!rm->rank_lens || rm->this_rank < 0 || rm->this_rank > num_extra)
+      return fail(FD_ERR_INVALID_ARG, "fd_combine: rank_merge needs rank_lens and 0 <= this_rank %d <= num_extra %d",
+                  rm->this_rank, num_extra);
+    a.rank_lens = rm->rank_lens;
+    a.this_rank = rm->this_rank;
+    if (rm->local_out) {
+      if (!dtype_size(rm->local_dtype) || rm->local_dtype == FD_FP8_E4M3)
+        return fail(FD_ERR_UNSUPPORTED, "fd_combine: rank_merge.local_dtype %d", rm->local_dtype);
+      if ((int64_t)num_partials + num_extra > 1024)
+        return fail(FD_ERR_TOO_LARGE, "fd_combine: rank_merge.local_out with more than 1024 partials");
+      a.local_out = rm->local_out;
+      a.local_dtype = rm->local_dtype;
+      a.s_lb = rm->stride_lb;
+      a.s_lh = rm->stride_lh;
+    }
   }
   int rc = fd_launch_combine((hipStream_t)stream, a);
   if (rc != FD_OK) return fail(rc, "fd_combine: launch failed: %s", hipGetErrorString(hipGetLastError()));

@@ -61,7 +61,13 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   }
   // LSE of partial s, -inf when the partial is not valid
   auto partial_lse = [&](int s) -> float {
-    if (s >= S) return a.extra_lse[((int64_t)(s - S) * a.batch + b) * a.Hq + h];  // extras: always valid
+    if (s >= S) {   // extras: always valid, unless they stand for other ranks whose lengths say otherwise
+      if (a.rank_lens) {
+        const int e = s - S;
+        if (a.rank_lens[(int64_t)(e < a.this_rank ? e : e + 1) * a.batch + b] <= 0) return -INFINITY;
+      }
+      return a.extra_lse[((int64_t)(s - S) * a.batch + b) * a.Hq + h];
+    }
     if (a.mode == FD_COMBINE_RANK) {
       if (a.seqlens[(int64_t)s * a.batch + b] <= 0) return -INFINITY;
     } else if (!own && (int64_t)per * s >= kv_len) {  // empty split range
@@ -104,6 +110,11 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float M = -INFINITY;  // running max over the passes (one pass unless NP > kMaxPartials)
   float L = 0.f;        // sum of the weights of this thread's rows
+  // local_out: the merge of the S split partials alone goes there as well (this rank's slot of a staged buffer), with
+  // weights relative to the maximum over those S, so that a far larger LSE among the extras cannot flush them to zero
+  const bool two = a.local_out != nullptr;   // (the host admits it only with NP <= kMaxPartials: one pass)
+  f32x4 acc_loc = {0.f, 0.f, 0.f, 0.f};
+  float M_loc = -INFINITY, L_loc = 0.f;
 
   if (own && NP <= ROWS * kPrefetch) {
     // one dependent round trip: the rows are requested together with the LSEs
@@ -116,13 +127,19 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
     for (int i = tid; i < NP; i += kCombineThreads) s_lse[i] = partial_lse(i);
     __syncthreads();
     M = wave_max_of(s_lse, NP);
+    if (two) M_loc = wave_max_of(s_lse, S);
     if (M > -INFINITY) {
 #pragma unroll
       for (int p = 0; p < kPrefetch; ++p) {
         const int s = r + p * ROWS;
         const float wgt = s < NP ? __expf(s_lse[s] - M) : 0.f;
-        acc += pre[p] * wgt;
+        if (wgt != 0.f) acc += pre[p] * wgt;   // (the row of an extra that does not count may hold anything)
         L += wgt;
+        if (two && s < S && M_loc > -INFINITY) {
+          const float wl = __expf(s_lse[s] - M_loc);
+          acc_loc += pre[p] * wl;
+          L_loc += wl;
+        }
       }
     }
   } else {
@@ -138,17 +155,19 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
       acc *= resc;
       L *= resc;
       M = m_new;
+      if (two) M_loc = wave_max_of(s_lse, min(cnt, S));
       for (int i = r; i < cnt; i += ROWS) {
         const float wgt = __expf(s_lse[i] - M);
-        if (wgt == 0.f) continue;
-        acc += load_row(p0 + i) * wgt;
+        const float wl = two && i < S && M_loc > -INFINITY ? __expf(s_lse[i] - M_loc) : 0.f;
+        if (wgt == 0.f && wl == 0.f) continue;
+        const f32x4 row = load_row(p0 + i);
+        if (wgt != 0.f) acc += row * wgt;
         L += wgt;
+        if (wl != 0.f) acc_loc += row * wl;
+        L_loc += wl;
       }
     }
   }
-  *(f32x4*)&s_acc[tid * 4] = acc;   // row r, columns 4 * (tid % CG) .. + 3 of the chunk
-  if ((tid & (CG - 1)) == 0) s_l[r] = L;
-  __syncthreads();
   // Sum over the ROWS row groups in two short steps instead of one thread per column walking all of them (64 dependent
   // LDS reads for a 16-column chunk): thread (g, col) adds the four rows g, g + NG, g + 2 NG, g + 3 NG of its column
   // (ROWS = 4 NG), the NG sums of a column go back through LDS, and the sum of the weights is a butterfly over one wave.
@@ -156,28 +175,40 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
   const int NG = kCombineThreads / ncol;        // = ROWS / 4
   const int col = tid & (ncol - 1);
   const int g = tid >> (a.cg_shift + 2);
-  float part4 = 0.f;
+  // dst / dst_base / dst_dtype: the output row; lse_col: the LSE goes to column D of it; lse_sep: and / or there
+  auto reduce_store = [&](const f32x4 acc_t, const float L_t, const float M_t, void* dst, int64_t dst_base, int dst_dtype,
+                          bool lse_col, float* lse_sep) {
+    *(f32x4*)&s_acc[tid * 4] = acc_t;   // row r, columns 4 * (tid % CG) .. + 3 of the chunk
+    if ((tid & (CG - 1)) == 0) s_l[r] = L_t;
+    __syncthreads();
+    float part4 = 0.f;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) part4 += s_acc[(g + k * NG) * ncol + col];
-  float lw = (tid & 63) < ROWS ? s_l[tid & 63] : 0.f;   // ROWS <= 64
+    for (int k = 0; k < 4; ++k) part4 += s_acc[(g + k * NG) * ncol + col];
+    float lw = (tid & 63) < ROWS ? s_l[tid & 63] : 0.f;   // ROWS <= 64
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) lw += __shfl_xor(lw, off);
-  __syncthreads();
-  s_acc[g * ncol + col] = part4;
-  __syncthreads();
-  if (tid < ncol) {
-    float o = 0.f;
-    for (int i = 0; i < NG; ++i) o += s_acc[i * ncol + tid];
-    const float Lsum = lw;
-    const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
-    const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
-    store_from_f32(a.out, out_base + col0 + tid, a.out_dtype, o * inv);
-    if (tid == 0 && col0 == 0) {
-      const float lse = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
-      if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, lse);
-      if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = lse;
+    for (int off = 32; off > 0; off >>= 1) lw += __shfl_xor(lw, off);
+    __syncthreads();
+    s_acc[g * ncol + col] = part4;
+    __syncthreads();
+    if (tid < ncol) {
+      float o = 0.f;
+      for (int i = 0; i < NG; ++i) o += s_acc[i * ncol + tid];
+      const float Lsum = lw;
+      const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+      store_from_f32(dst, dst_base + col0 + tid, dst_dtype, o * inv);
+      if (tid == 0 && col0 == 0) {
+        const float lse = Lsum > 0.f ? M_t + __logf(Lsum) : -INFINITY;
+        if (lse_col) store_from_f32(dst, dst_base + D, dst_dtype, lse);
+        if (lse_sep) *lse_sep = lse;
+      }
     }
+  };
+  if (two) {
+    reduce_store(acc_loc, L_loc, M_loc, a.local_out, (int64_t)b * a.s_lb + (int64_t)h * a.s_lh, a.local_dtype, true, nullptr);
+    __syncthreads();
   }
+  reduce_store(acc, L, M, a.out, (int64_t)b * a.s_ob + (int64_t)h * a.s_oh, a.out_dtype, a.mode == FD_COMBINE_SPLIT_LSE,
+               a.lse_out ? a.lse_out + (int64_t)b * a.Hq + h : nullptr);
 }
 
 // Up to MAXP (16, 32 or 64) partials produced by this library's split kernel in the same call, rows readable four
@@ -313,7 +344,7 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   // 32 only where there is a workgroup per CU: with few output rows (one long sequence: 96 rows x 42 partials) the
   // general kernel, which spreads a row over several workgroups, is the faster one (5.0 against 5.7 us)
   const int np_own = a.num_partials <= 16 ? 16 : (a.num_partials <= 32 ? 32 : 64);
-  const bool small = (a.all_slots_written || a.mode == FD_COMBINE_RANK) && a.num_extra == 0 &&
+  const bool small = (a.all_slots_written || a.mode == FD_COMBINE_RANK) && a.num_extra == 0 && !a.local_out &&
                      (a.num_partials <= 32 || (a.num_partials <= 64 && rows >= 256));
   // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
   // one workgroup per CU and a thread would still have more than two partials to walk.

@@ -106,6 +106,12 @@ struct CombineArgs {
                               // writes every slot (empty splits as out = 0, lse = -inf)
   int64_t capacity;           // split modes: lengths are clamped to it, as the split kernels clamp them to the block
                               // table's capacity (stand-alone calls that do not know a table: 2^31 - 1 - num_partials)
+  // fd_rank_merge: the extras stand for the other ranks of a sequence-parallel decode
+  const int32_t* rank_lens;   // nullptr, or [num_extra + 1, batch]: extra e counts iff its rank's length is > 0
+  int32_t this_rank;          // the row of rank_lens that is not an extra
+  int32_t local_dtype;
+  void* local_out;            // nullptr, or [batch, Hq, D + 1]: the merge of the split partials alone, LSE at column D
+  int64_t s_lb, s_lh;
 };
 
 // How a decode step cuts a sequence into ranges: what the scheduler needs to know of it.

@@ -31,6 +31,11 @@ Keyword-only additions that the reference does not have (all default off):
   no_alloc        True: the split partials live in the library's static device array (``fd_decode_noalloc``, at most
                   16 MiB of them) and the call allocates nothing -- for steps captured into a HIP graph or run where
                   allocation is not allowed; needs ``output_combine``; calls that overlap on one GPU must not share it
+  rank_merge      ``(global_kv_lens [R, B] int32, this_rank, local_out or None)`` with ``extra_partials`` of the R - 1
+                  other ranks in rank order: the combine treats the extras as those ranks' partials -- rank r counts for
+                  sequence b iff ``global_kv_lens[r, b] > 0`` (flash_decode.py:513-515) -- and also writes the merge of
+                  the local splits alone, LSE in the last column, to ``local_out [B, Hq, Dv + 1]``: intra-rank
+                  combine, staging copy and inter-rank combine of the sequence-parallel layer in one launch
   fuse_combine    True: one launch, the combine runs in the tail of the split kernel (pays off when
                   the groups of a ragged batch finish at different times, or for very short steps launched
                   eagerly, where the second launch's host time counts); False (default): split kernel and
@@ -47,7 +52,7 @@ use).
 """
 from __future__ import annotations
 
-from ctypes import byref
+from ctypes import addressof, byref
 from typing import Optional
 
 import torch
@@ -55,7 +60,7 @@ import torch
 from .._lib import (FD_COMBINE_RANK, FD_COMBINE_SPLIT, FD_COMBINE_SPLIT_LSE, FD_F32, FD_NOALLOC_SCRATCH_BYTES,
                     FD_ORDER_ITEMS, FD_ORDER_SEQUENCES, FD_PATH_AUTO, FD_PATH_MFMA, FD_PATH_VALU,
                     FD_STEP_CALLER_PARTIALS, FD_STEP_EXACT_SPLITS, FD_STEP_FUSED, FD_STEP_LSE_TWICE, FD_STEP_NO_ORDER,
-                    FD_STEP_SCHEDULE, FdDecodeArgs, FdLaunchPlan, FdParams, check, fd_dtype_of, load_library,
+                    FD_STEP_SCHEDULE, FdDecodeArgs, FdLaunchPlan, FdParams, FdRankMerge, check, fd_dtype_of, load_library,
                     stream_handle)
 
 _PATHS = {"auto": FD_PATH_AUTO, "valu": FD_PATH_VALU, "mfma": FD_PATH_MFMA}
@@ -228,7 +233,7 @@ _STEP_CACHE = {}   # fd_decode_args images of planned steps by everything but th
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
             seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
-            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False, auto_order=True):
+            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False, auto_order=True, rank_merge=None):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     v_shape = v_cache.shape
@@ -264,6 +269,21 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         assert ex_lse.is_contiguous() and ex_out.dtype == output_combine.dtype
     if lse_out is not None:
         assert lse_out.dtype == torch.float32 and lse_out.is_contiguous() and lse_out.numel() == batch * q_heads
+    rm = None
+    if rank_merge is not None:
+        # sequence-parallel decode: the extras stand for the other ranks (fd_rank_merge)
+        rank_lens, this_rank, local_out = rank_merge
+        _require_cuda(rank_lens, local_out)
+        assert rank_lens.dtype == torch.int32 and rank_lens.is_contiguous()
+        assert tuple(rank_lens.shape) == (n_extra + 1, batch) and 0 <= this_rank <= n_extra
+        if fuse_combine:
+            raise RuntimeError("rank_merge is not available with fuse_combine")
+        rm = FdRankMerge()
+        rm.rank_lens, rm.this_rank = rank_lens.data_ptr(), this_rank
+        if local_out is not None:
+            assert tuple(local_out.shape) == (batch, q_heads, v_head_dim + 1) and local_out.stride(2) == 1
+            rm.local_out, rm.local_dtype = local_out.data_ptr(), fd_dtype_of(local_out)
+            rm.stride_lb, rm.stride_lh = local_out.stride(0), local_out.stride(1)
     if seq_order_lens is not None:
         assert seq_order is not None and seq_order_lens.dtype == torch.int32 and seq_order_lens.is_contiguous()
         assert seq_order_lens.numel() == batch
@@ -323,6 +343,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             a.extra_out, a.extra_lse = ex_out.data_ptr(), ex_lse.data_ptr()
         if k_scale is not None:
             a.params.k_scale, a.params.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
+        if rm is not None:
+            a.params.rank_merge = addressof(rm)
         rc = lib.fd_decode_planned(hstream, byref(a))
         if rc:
             check(rc)
@@ -397,6 +419,8 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         p.seq_order_lens = None
         seq_order = item_order
     mode = FD_COMBINE_SPLIT_LSE if with_lse_column else FD_COMBINE_SPLIT
+    if rm is not None:
+        p.rank_merge = addressof(rm)
     if no_alloc:
         check(lib.fd_decode_noalloc(
             hstream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output_combine.data_ptr(),

@@ -14,12 +14,18 @@ reference's:
      ``global_kv_lens[r, b] > 0``                   (:173-183)
 
 Step 2 is where the reference allgathers over NVSHMEM (:139).  Nothing here
-spans more than one GPU: the other ranks' slots are filled from
+spans more than one GPU: the other ranks' partials come from
 ``remote_partials`` -- ``(out [R-1, B, Hq, Dv], lse [R-1, B, Hq])`` in rank order
-with this rank left out -- which the caller produces on the same device.  With
-``num_ranks == 1`` no remote partials are needed and steps 2 and 3 fall away: the local decode writes the final output.  The staged slots keep the
-layout a push-allgather would write into, so one can be put in front of step 3
-later without touching the kernels.
+with this rank left out -- which the caller produces on the same device.  By
+default a forward is two launches: the split kernel and one combine that merges
+the local splits, writes that merge into this rank's slot (the slot a push to
+the other ranks would be sent from) and merges it with the remote partials
+where they are.  ``staged_exchange=True`` walks the reference's steps one by
+one instead -- local result into its slot, the others' partials copied into
+theirs, stand-alone inter-rank kernel over the slots -- which is the shape a
+real exchange would take: a push-allgather writes the slots, step 3 follows.
+With ``num_ranks == 1`` no remote partials are needed and steps 2 and 3 fall
+away: the local decode writes the final output.
 
 The staged partials are fp32 by default, so the LSE is not rounded to the
 query's 16-bit dtype as in the reference (:95-97); pass ``partial_dtype=q.dtype``
@@ -39,7 +45,7 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
 
     def __init__(self, rank, node, num_ranks, num_nodes, num_q_heads, num_kv_heads, q_head_dim, v_head_dim,
                  page_size=1, scale=1, soft_cap=0, max_allowed_batch=1, thrink_buffer_threshold=500, stages=20,
-                 partial_dtype: Optional[torch.dtype] = torch.float32):
+                 partial_dtype: Optional[torch.dtype] = torch.float32, staged_exchange: bool = False):
         super().__init__()
         self.rank = rank
         self.num_ranks = num_ranks
@@ -60,6 +66,10 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         self.max_allowed_batch = max_allowed_batch
         self.stages = stages
         self.partial_dtype = partial_dtype
+        # False: the other ranks' partials are merged where the caller holds them (two launches per forward);
+        # True: they are first copied into their slots of the staged buffer and merged from there by the stand-alone
+        # inter-rank kernel, step by step as in the reference
+        self.staged_exchange = staged_exchange
         assert 0 <= rank < num_ranks
 
         # staging ring for the gathered partials (a plain device tensor: no symmetric heap on one GPU)
@@ -129,24 +139,38 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         stage = self._stage(nbytes_per_rank * self.num_ranks, q.device)
         all_ranks_output_combine = stage.view(pdtype).view([self.num_ranks, batch, self.num_q_heads, d1])
         final_output = torch.empty([batch, self.num_q_heads, self.v_head_dim], dtype=q.dtype, device=q.device)
+        r_out, r_lse = remote_partials
+        assert r_out.shape[0] == self.num_ranks - 1 and r_lse.shape[0] == self.num_ranks - 1
 
-        # local decode straight into this rank's slot (the reference copies it there, :136-138)
+        if not self.staged_exchange:
+            # Two launches: the split kernel, and ONE combine that does what the reference does in three steps -- the
+            # intra-rank combine (:107-110), the copy of its result into this rank's slot of the staged buffer
+            # (:136-138: the slot a push to the other ranks would be sent from) and the inter-rank combine (:173-183),
+            # reading the other ranks' partials where the caller holds them instead of from their slots; rank r
+            # counts for sequence b iff global_kv_lens[r, b] > 0, as in the reference's kernel.
+            gqa_fwd_batch_decode(q, k_cache, v_cache, self.workspace, None, global_kv_lens[self.rank], block_table,
+                                 self.scale, soft_cap=self.soft_cap, output_split=output_split,
+                                 output_combine=final_output, kv_split=self.kv_split,
+                                 extra_partials=(r_out, r_lse),
+                                 rank_merge=(global_kv_lens, self.rank, all_ranks_output_combine[self.rank]))
+            self.signal_target += 1
+            return final_output
+
+        # The reference's own sequence of steps, slot by slot (what a real exchange would feed): local decode straight
+        # into this rank's slot (the reference copies it there, :136-138) ...
         gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch, global_kv_lens[self.rank],
                                         block_table, self.scale, soft_cap=self.soft_cap,
                                         output_split=output_split,
                                         output_combine=all_ranks_output_combine[self.rank], kv_split=self.kv_split)
 
-        # stand-in for the allgather: the other ranks' partials arrive from the caller
-        if self.num_ranks > 1:
-            r_out, r_lse = remote_partials
-            assert r_out.shape[0] == self.num_ranks - 1 and r_lse.shape[0] == self.num_ranks - 1
-            others = [r for r in range(self.num_ranks) if r != self.rank]
-            for i, r in enumerate(others):
-                all_ranks_output_combine[r, :, :, :self.v_head_dim].copy_(r_out[i])
-                all_ranks_output_combine[r, :, :, self.v_head_dim].copy_(r_lse[i])
+        # ... stand-in for the allgather: the other ranks' partials arrive from the caller ...
+        others = [r for r in range(self.num_ranks) if r != self.rank]
+        for i, r in enumerate(others):
+            all_ranks_output_combine[r, :, :, :self.v_head_dim].copy_(r_out[i])
+            all_ranks_output_combine[r, :, :, self.v_head_dim].copy_(r_lse[i])
         self.signal_target += 1
 
-        # final combine, launched as the reference launches its Triton kernel
+        # ... and the final combine, launched as the reference launches its Triton kernel
         kernel_inter_rank_gqa_fwd_batch_decode_combine_kv[(batch, self.num_q_heads, 1)](
             all_ranks_output_combine,
             final_output,

@@ -27,7 +27,8 @@ class FdParams(Structure):            # struct fd_params, include/flash_decode.h
                 ("soft_cap", c_float), ("k_scale", c_void_p), ("v_scale", c_void_p),
                 ("path", c_int32), ("waves_per_block", c_int32), ("seq_order_lens", c_void_p),
                 ("split_align", c_int32), ("split_adapt", c_int32),
-                ("max_kv_len", c_int32), ("seq_order_items", c_int32), ("v_head_dim", c_int32)]
+                ("max_kv_len", c_int32), ("seq_order_items", c_int32), ("v_head_dim", c_int32),
+                ("rank_merge", c_void_p)]
 
 class FdDecodeArgs(Structure):        # struct fd_decode_args, include/flash_decode.h
     _fields_ = [("q", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p), ("workspace", c_void_p),
