@@ -44,6 +44,9 @@ def parse_args():
                     help="override the workload's kv_split (experiments); -1: the library's own choice")
     ap.add_argument("--exact-splits", action="store_true",
                     help="use exactly the workload's kv_split splits instead of the library's plan (fd_plan_splits)")
+    ap.add_argument("--caller-partials", default=None, choices=["fp32", "fp16", "bf16"],
+                    help="the caller hands in output_split [B, Hq, S, D + 1] of this type, as the reference's perf "
+                         "scripts and its sequence-parallel layer do: exactly kv_split observable partials")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-targets", action="store_true",
@@ -436,8 +439,9 @@ def main():
     algo_bytes = wl_cpu.algorithmic_bytes()
 
     pools = make_pools(torch, wl, dev, args.pools)
+    caller_dt = {None: None, "fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}[args.caller_partials]
     step, out, lse, workspace = make_step(torch, fd, wl, pools, S, dev, variant=args.variant, exact=args.exact_splits,
-                                          path=args.path, waves=args.waves, fuse=args.fuse)
+                                          path=args.path, waves=args.waves, fuse=args.fuse, caller_partials=caller_dt)
 
     # ---- whole-step timing
     ramp_ms = settle(torch, step, args.clock_ramp_ms)
@@ -482,8 +486,9 @@ def main():
     L = fd._lib
     # the plan the step above ran with (fd_plan_decode), so that this leg launches the same split kernel
     flags = (L.FD_STEP_EXACT_SPLITS if args.exact_splits else 0) | (L.FD_STEP_SCHEDULE if args.variant == "persistent" else 0) \
-        | (L.FD_STEP_FUSED if args.fuse else 0)
+        | (L.FD_STEP_FUSED if args.fuse else 0) | (L.FD_STEP_CALLER_PARTIALS if caller_dt is not None else 0)
     plan = fk.decode_plan(wl.q, wl.k_cache, wl.block_table, S, flags=flags, out_dtype=L.fd_dtype_of(out),
+                          mid_dtype=L.FD_F32 if caller_dt is None else L.fd_dtype_of(torch.empty(0, dtype=caller_dt)),
                           fp8=wl.k_scale is not None, path=args.path, waves_per_block=args.waves,
                           num_extra=0 if wl.extra_out is None else wl.extra_out.shape[0])
     S_eff = plan.num_splits
@@ -493,6 +498,10 @@ def main():
     split_ws = torch.empty(B * Hq * S_eff * (D + 1), dtype=torch.float32, device=dev)
     mid = split_ws[:n_o].view(B, Hq, S_eff, D)
     lse_split = split_ws[n_o:n_o + B * Hq * S_eff].view(B, Hq, S_eff)
+    lse_split_ptr = lse_split.data_ptr()
+    if caller_dt is not None:   # the reference's layout: rows of D + 1 elements, the LSE in the last one
+        mid = torch.empty(B, Hq, S_eff, D + 1, dtype=caller_dt, device=dev)
+        lse_split_ptr = None
     hstream = torch.cuda.current_stream().cuda_stream
     order_ptr = None
     if plan.order_kind == L.FD_ORDER_ITEMS:
@@ -508,7 +517,7 @@ def main():
     def split_only(i):
         k, v = pools[i % len(pools)]
         fd._lib.check(lib.fd_split_kv(
-            hstream, wl.q.data_ptr(), k.data_ptr(), v.data_ptr(), mid.data_ptr(), lse_split.data_ptr(),
+            hstream, wl.q.data_ptr(), k.data_ptr(), v.data_ptr(), mid.data_ptr(), lse_split_ptr,
             float(wl.scale), wl.block_table.data_ptr(), wl.kv_lens.data_ptr(), B,
             wl.q.stride(0), wl.q.stride(1), k.stride(-3), k.stride(-2), v.stride(-3), v.stride(-2),
             mid.stride(0), mid.stride(1), mid.stride(2), wl.block_table.stride(0), order_ptr, byref(p)))
@@ -577,7 +586,8 @@ def main():
                                        order_kind=["none", "sequences", "items"][plan.order_kind],
                                        workspace_bytes=plan.workspace_bytes),
                    "kv_len_total": int(wl_cpu.kv_lens.sum()), "kv_pools_rotated": len(pools),
-                   "variant": args.variant, "path": args.path, "fused_combine": args.fuse},
+                   "variant": args.variant, "path": args.path, "fused_combine": args.fuse,
+                   "caller_partials": args.caller_partials},
         "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
@@ -610,7 +620,8 @@ def main():
                           "frac_of_dense_bf16_peak": round(issued / (split_us * 1e-6) / 2.5e15, 4)}
 
     headline = args.config == 2 and not args.shape and not args.bf16_twin and args.variant == "plain" \
-        and not args.exact_splits and args.path == "auto" and not args.fuse and not args.kv_split
+        and not args.exact_splits and args.path == "auto" and not args.fuse and not args.kv_split \
+        and not args.caller_partials
     targets = None
     if headline and not args.no_targets:
         targets = measure_targets(torch, fd, dev, args.steps, args.warmup, (wl, pools))

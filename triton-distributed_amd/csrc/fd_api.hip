@@ -105,8 +105,7 @@ constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged b
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
 constexpr int64_t kStoreThroughBytes = 16 << 20;   // partials of a step from which on they are written through
 constexpr int kMaxChunkBatch = 32;     // chunked work items: largest batch they are used for
-constexpr int kMaxSplitsPerWave = 2;   // chunked work items: splits one wave walks (all but the last parked in LDS)
-constexpr int kMaxSplitsPerWaveFinal = 4;   // ... when a parked partial is the finished one (a quarter to an eighth of the bytes)
+constexpr int kMaxSplitsPerWave = 4;   // chunked work items: splits one wave walks (finished partials parked in LDS)
 constexpr int kChunkLdsBytes = 80 * 1024;   // LDS a chunked workgroup may take: two of them per CU
 
 int env_waves() {
@@ -354,11 +353,9 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   // the fp8 head_dim-64 kernel keeps 8 KB in flight per wave with one KV head per wave, like the VALU kernel;
   // the other MFMA kernels 16 KB
   const int64_t wave_target = use_mfma && !(kv_fp8 && D == 64 && !pair) ? kTargetWaves : kTargetWavesValu;
-  // Partials with rows on multiples of four elements (the library's own layout) are parked finished -- normalised,
-  // in mid_dtype, the rows of the real heads only: 2 KB for 8 heads in bf16 against 8.3 KB of raw state -- and a
-  // wave walks up to four splits; else the raw state is parked and normalised when it is stored.
+  // Partials are parked finished -- normalised, in mid_dtype, the rows of the real heads only: 2 KB for 8 heads in
+  // bf16 against 8.3 KB of raw state -- and a wave walks up to four splits.
   const int hb_slots = a.hbsz > 16 ? 32 : 16;
-  const bool park_final = a.vec_out != 0;
   // What a wish of `wish` consecutive splits per work item becomes: the waves of a head take whole splits,
   // kMaxSplitsPerWave at most -- a wave keeps the finished partials of all but its last split in LDS until it has
   // issued its last load (stores and loads of a wave retire in order, so a store between two tiles would hold back
@@ -395,8 +392,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
     if (wish > 1) {
       while (c.waves > 1 && c.waves > wish) c.waves >>= 1;
       c.per_wave = round_up ? (wish + c.waves - 1) / c.waves : wish / c.waves;
-      const int cap = park_final ? kMaxSplitsPerWaveFinal : kMaxSplitsPerWave;
-      if (c.per_wave > cap) c.per_wave = cap;
+      if (c.per_wave > kMaxSplitsPerWave) c.per_wave = kMaxSplitsPerWave;
       c.chunk = c.waves * c.per_wave;
     }
     c.grid_waves = (int64_t)batch * ((a.S + c.chunk - 1) / c.chunk) * a.Hkv * a.nhb * c.waves;
@@ -429,8 +425,7 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   int waves = cp.waves;
   int chunk_per_wave = cp.per_wave;
   if (a.chunk > 1) {
-    a.park_final = park_final;
-    a.park_bytes = a.park_final ? hb_slots * 4 + a.hbsz * D * msz : (hb_slots * D + 2 * hb_slots) * 4;
+    a.park_bytes = hb_slots * 4 + a.hbsz * D * msz;
     a.park = chunk_per_wave - 1;
   }
   // Heads per workgroup: only the MFMA kernels, and not with the fused combine (its tickets are per KV head).

@@ -66,15 +66,14 @@ struct SplitArgs {
   int32_t store_through;          // 1: partials are written through to memory (sc0 sc1) instead of being left dirty in
                                   // the XCD's L2 until the kernel ends; pays off for tens of MB of partials
   int32_t park;                   // chunked work items: finished partials a wave parks in LDS besides its last one
+                                  // (which goes to the wave's tile staging buffer)
   // V head dim != K head dim on the head_dim-128 MFMA kernel.  dv = V head dim (the column of an in-row LSE).
   // v_members = 2 (dv 256): a workgroup member is a (KV head, 128-column half of the V rows) pair -- two waves share
   // K and the softmax and each accumulates and stores its own half.  v_chunk_mask = 7 (dv 64): the 16 lanes of a
   // wave row fetch the eight 16-byte chunks of a 128-byte V row twice, and only v_cols = 64 columns are stored.
   int32_t dv, v_members, v_chunk_mask, v_cols;
-  int32_t park_final;             // 1: a parked partial is the finished one -- fp32 LSEs of the wave's head slots, then
-                                  // normalised rows [head][D] in mid_dtype (rows that start on multiples of four
-                                  // elements only); 0: the wave's raw state in cta_merge_store's layout
-  int32_t park_bytes;             // LDS bytes of one parked partial
+  int32_t park_bytes;             // LDS bytes of one parked partial: the finished one -- fp32 LSEs of the wave's head
+                                  // slots, then the normalised rows [head][D] of its real heads in mid_dtype
   // Fused combine (tickets != nullptr): the workgroup that finishes a (sequence, head block) last
   // merges its S partials (+ num_extra further ones) into the final output.
   int32_t* tickets;      // one zero-initialised counter per (sequence, KV head, head block); left at zero
@@ -237,8 +236,7 @@ __device__ __forceinline__ void store_partial4(void* base, int64_t off, int dtyp
   }
 }
 
-// One value, or two adjacent 16-bit values as one dword (off even, base 4-byte aligned), with the same write-through
-// option and the same restriction as store_partial4.
+// One value, with the same write-through option and the same restriction as store_partial4.
 __device__ __forceinline__ void store_partial1(void* base, int64_t off, int dtype, float x, bool through) {
   if (!through) { store_from_f32(base, off, dtype, x); return; }
   if (dtype == FD_F32) {
@@ -249,18 +247,6 @@ __device__ __forceinline__ void store_partial1(void* base, int64_t off, int dtyp
     asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"((uint16_t*)base + off), "v"(w) : "memory");
   }
 }
-__device__ __forceinline__ void store_partial2x16(void* base, int64_t off, int dtype, float x0, float x1, bool through) {
-  const f32x2 v = {x0, x1};
-  const uint32_t w = dtype == FD_F16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2))
-                                     : __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-  uint16_t* p = (uint16_t*)base + off;
-  if (through) {
-    asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
-  } else {
-    *(uint32_t*)p = w;
-  }
-}
-
 // Orders LDS accesses of one wave: lanes of a wave exchange data through LDS
 // without a workgroup barrier (the LDS queue of a wave is in order); this only
 // stops the compiler from moving accesses across the point.
@@ -801,171 +787,206 @@ __device__ __forceinline__ void park_store8(char* rows, int elem, int dtype, con
   }
 }
 
-// Chunked work items, SplitArgs::park_final: ONE wave copies a finished partial that it parked in LDS (HB fp32 LSEs,
-// then rows [head][D] in mid_dtype) to split s of its head slots.  Same geometry as wave_store_partial: four values
-// per lane, whole rows per store instruction.
+// Raw-bit stores of one dword / one 16-bit value, optionally written through (same restriction as store_partial4).
+__device__ __forceinline__ void store_bits32(void* p, uint32_t w, bool through) {
+  if (through) {
+    asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+  } else {
+    *(uint32_t*)p = w;
+  }
+}
+__device__ __forceinline__ void store_bits16(void* p, uint32_t w, bool through) {
+  if (through) {
+    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+  } else {
+    *(uint16_t*)p = (uint16_t)w;
+  }
+}
+__device__ __forceinline__ uint32_t f32_to_bits16(float x, int dtype) {
+  return dtype == FD_F16 ? (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x)
+                         : (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
+}
+
+// Chunked work items: ONE wave copies a finished partial that it parked in LDS (HB fp32 LSEs, then the normalised
+// rows [head][D] of its real heads in mid_dtype) to split s of its head slots.  Called at the end of the wave's run
+// only: on this target stores and loads of a wave retire in order (one vmcnt), so a store issued between two tiles
+// would hold back every later K/V load until it is acknowledged.  empty: the split holds no token (out = 0,
+// lse = -inf; the slot is not read).
+//  * Rows that start on multiples of four elements (the library's own layout): four values per lane, whole rows per
+//    store instruction.
+//  * Else (the reference's [B, Hq, S, D + 1] layout, whose rows are D + 1 elements apart): consecutive lanes on
+//    consecutive elements, so that a store instruction still covers contiguous memory.  A 16-bit row of D values with
+//    the LSE behind them goes out as dwords of two values on 4-byte boundaries: a row that starts between two
+//    boundaries stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that starts on a boundary pairs (0, 1) ..
+//    (D - 2, D - 1) and stores the LSE alone.  The values are the parked bits: nothing is scaled or converted here
+//    but the LSE, and every LDS read of four rows is requested before the first store.
 template <int HB, int D>
 __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char* slot, int b, int head0, int nheads,
-                                                 int s) {
+                                                 int s, bool empty) {
   const int lane = threadIdx.x & 63;
   constexpr int D4 = D / 4;
   constexpr int RPI = 64 / D4;
+  static_assert(D4 <= 64 && HB % RPI == 0 && D % 128 == 0, "one wave covers whole rows");
   const float* lse_slot = (const float*)slot;
   const char* rows = slot + HB * 4;
-  const int d = (lane % D4) * 4;
   const bool through = a.store_through != 0;
+  if (a.vec_out) {
+    const int d = (lane % D4) * 4;
 #pragma unroll
-  for (int r = 0; r < HB / RPI; ++r) {
-    const int h = r * RPI + lane / D4;
-    if (h >= nheads) continue;
-    const int head = head0 + h;
-    const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
-    if (a.mid_dtype == FD_F32) {
-      const f32x4 v = *(const f32x4*)((const float*)rows + h * D + d);
-      float* p = (float*)a.out + off;
-      if (through) {
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-      } else {
-        *(f32x4*)p = v;
-      }
-    } else {
-      const u32x2 v = *(const u32x2*)((const uint16_t*)rows + h * D + d);
-      uint16_t* p = (uint16_t*)a.out + off;
-      if (through) {
-        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
-      } else {
-        *(u32x2*)p = v;
-      }
-    }
-    if (d == 0 && !a.no_lse) {
-      const float lse = lse_slot[h];
-      if (a.lse) {
-        a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
-      } else {
-        store_partial1(a.out, off + D, a.mid_dtype, lse, through);
-      }
-    }
-  }
-}
-
-// Values one lane holds of a D-wide row in wave_store_partial's element-wise forms: 64 lanes x 1 value (or x 2 values
-// for the 16-bit pairs) per pass.
-template <int D>
-__host__ __device__ constexpr int paired_values_per_lane() { return D <= 128 ? 2 : D / 64; }
-
-// Chunked work items: ONE wave stores the finished partial of split s for its own HB head slots, from an LDS buffer
-// `part` of its own (same layout as one wave's slice in cta_merge_store; the wave has ordered its LDS writes before
-// the call).  Called at the end of the wave's run only: on this target stores and loads of a wave retire in order
-// (one vmcnt), so a store issued between two tiles would hold back every later K/V load until it is acknowledged.  Rows are read back row-major, so a store instruction covers whole 512-byte rows.  empty: the split holds no
-// token (out = 0, lse = -inf; `part` is not read).
-template <int HB, int D>
-__device__ __forceinline__ void wave_store_partial(const SplitArgs& a, const float* part, int b, int head0, int nheads,
-                                                   int s, bool empty) {
-  const int lane = threadIdx.x & 63;
-  constexpr int D4 = D / 4;          // lanes per row
-  constexpr int RPI = 64 / D4;       // rows per store instruction
-  static_assert(D4 <= 64 && HB % RPI == 0, "one wave covers whole rows");
-  if (!a.vec_out) {
-    // Rows that do not start on a multiple of four elements (the reference's D + 1 layout): consecutive lanes on
-    // consecutive elements, so that a store instruction covers contiguous memory.  A 16-bit row of D values with the
-    // LSE behind them goes out as dwords of two values on 4-byte boundaries: a row that starts between two boundaries
-    // stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that starts on a boundary pairs (0, 1) ..
-    // (D - 2, D - 1) and stores the LSE alone.
-    const bool through = a.store_through != 0;
-    const bool paired = a.mid_dtype != FD_F32 && !a.lse && !a.no_lse;
-    const int64_t row0 = (int64_t)b * a.so_b + (int64_t)head0 * a.so_h + (int64_t)s * a.so_s;
-    const uint64_t par0 = (reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row0;
-    // lane h holds row h's scale and LSE (one LDS round trip for all rows) and stores the row's single value
-    const int hl = lane < nheads ? lane : nheads - 1;
-    float inv_l = 0.f, lse_l = -INFINITY, x0_l = 0.f;
-    if (!empty) {
-      const float M = part[HB * D + hl];
-      const float L = part[HB * D + HB + hl];
-      inv_l = L > 0.f ? 1.0f / L : 0.f;
-      lse_l = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
-      x0_l = part[hl * D] * inv_l;
-    }
-    if (lane < nheads) {
-      const int64_t row_l = row0 + (int64_t)hl * a.so_h;
-      if (paired) {
-        const bool first_l = ((par0 + (uint64_t)hl * (uint64_t)a.so_h) & 1) != 0;
-        store_partial1(a.out, row_l + (first_l ? 0 : D), a.mid_dtype, first_l ? x0_l : lse_l, through);
-      } else if (!a.no_lse) {
-        if (a.lse) {
-          a.lse[((int64_t)b * a.Hq + head0 + hl) * a.S + s] = lse_l;
+    for (int r = 0; r < HB / RPI; ++r) {
+      const int h = r * RPI + lane / D4;
+      if (h >= nheads) continue;
+      const int head = head0 + h;
+      const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
+      if (a.mid_dtype == FD_F32) {
+        const f32x4 v = empty ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)((const float*)rows + h * D + d);
+        float* p = (float*)a.out + off;
+        if (through) {
+          asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
         } else {
-          store_partial1(a.out, row_l + D, a.mid_dtype, lse_l, through);
+          *(f32x4*)p = v;
+        }
+      } else {
+        const u32x2 v = empty ? u32x2{0u, 0u} : *(const u32x2*)((const uint16_t*)rows + h * D + d);
+        uint16_t* p = (uint16_t*)a.out + off;
+        if (through) {
+          asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+        } else {
+          *(u32x2*)p = v;
+        }
+      }
+      if (d == 0 && !a.no_lse) {
+        const float lse = empty ? -INFINITY : lse_slot[h];
+        if (a.lse) {
+          a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
+        } else {
+          store_partial1(a.out, off + D, a.mid_dtype, lse, through);
         }
       }
     }
-    // four rows at a time: their values are requested from LDS together
-    constexpr int NV = paired_values_per_lane<D>();
+    return;
+  }
+  const int64_t row0 = (int64_t)b * a.so_b + (int64_t)head0 * a.so_h + (int64_t)s * a.so_s;
+  // lane h serves row h's single values: its LSE (and, for paired 16-bit rows, the row's odd value)
+  const int hl = lane < nheads ? lane : nheads - 1;
+  const float lse_l = empty ? -INFINITY : lse_slot[hl];
+  if (a.mid_dtype == FD_F32) {
+    constexpr int NV = D / 64;
+    float* out = (float*)a.out;
     for (int h0 = 0; h0 < nheads; h0 += 4) {
-      float x[4][NV];
-      float inv[4], lse[4];
-      int first[4];
+      uint32_t x[4][NV];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int hh = min(h0 + i, nheads - 1);
-        inv[i] = __shfl(inv_l, hh);
-        lse[i] = __shfl(lse_l, hh);
-        first[i] = paired ? (int)((par0 + (uint64_t)hh * (uint64_t)a.so_h) & 1) : 0;
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-          // paired: values 2 (lane + 64 (k / 2)) + first + (k & 1); else lane + 64 k
-          const int e = paired ? 2 * (lane + 64 * (k >> 1)) + first[i] + (k & 1) : lane + 64 * k;
-          x[i][k] = empty || e >= D ? 0.f : part[hh * D + e];
+        for (int k = 0; k < NV; ++k) x[i][k] = empty ? 0u : ((const uint32_t*)rows)[hh * D + lane + 64 * k];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (h0 + i >= nheads) break;
+        float* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) store_bits32(row + lane + 64 * k, x[i][k], through);
+      }
+    }
+    if (lane < nheads && !a.no_lse) {
+      if (a.lse) {
+        a.lse[((int64_t)b * a.Hq + head0 + hl) * a.S + s] = lse_l;
+      } else {
+        store_bits32(out + row0 + (int64_t)hl * a.so_h + D, __float_as_uint(lse_l), through);
+      }
+    }
+    return;
+  }
+  uint16_t* out = (uint16_t*)a.out;
+  const uint16_t* r16 = (const uint16_t*)rows;
+  const uint32_t* r32 = (const uint32_t*)rows;
+  const uint32_t lse16_l = f32_to_bits16(lse_l, a.mid_dtype);
+  const bool paired = !a.lse && !a.no_lse;
+  if (!paired) {
+    // 16-bit rows without an LSE behind them: element by element
+    constexpr int NV = D / 64;
+    for (int h = 0; h < nheads; ++h) {
+      uint16_t* row = out + row0 + (int64_t)h * a.so_h;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) store_bits16(row + lane + 64 * k, empty ? 0u : r16[h * D + lane + 64 * k], through);
+    }
+    if (lane < nheads && !a.no_lse) a.lse[((int64_t)b * a.Hq + head0 + hl) * a.S + s] = lse_l;
+    return;
+  }
+  // element parity of a row's start relative to a 4-byte boundary
+  const uint64_t par0 = (reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row0;
+  constexpr int NW = D / 128;   // dwords per lane and row
+  if ((a.so_h & 1) == 0) {
+    // The usual case -- an even number of splits, so that all heads of a split start with the same parity: one
+    // wave-uniform decision instead of one per row.
+    const bool first = (__builtin_amdgcn_readfirstlane((int)(par0 & 1))) != 0;
+    if (lane < nheads) {
+      uint16_t* row = out + row0 + (int64_t)hl * a.so_h;
+      store_bits16(row + (first ? 0 : D), first ? (empty ? 0u : (uint32_t)r16[hl * D]) : lse16_l, through);
+    }
+    for (int h0 = 0; h0 < nheads; h0 += 4) {
+      uint32_t lo[4][NW], hi[4][NW], lse16[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int hh = min(h0 + i, nheads - 1);
+        if (first) lse16[i] = f32_to_bits16(empty ? -INFINITY : lse_slot[hh], a.mid_dtype);
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+          const int w = lane + 64 * k;   // dword of the parked row: values 2 w, 2 w + 1
+          lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
+          if (first) hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
         }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (h0 + i >= nheads) break;
-        const int64_t row = row0 + (int64_t)(h0 + i) * a.so_h;
-        if (paired) {
+        uint16_t* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
 #pragma unroll
-          for (int k = 0; k < NV; k += 2) {
-            const int e = 2 * (lane + 64 * (k >> 1)) + first[i];
-            if (e < D)
-              store_partial2x16(a.out, row + e, a.mid_dtype, x[i][k] * inv[i],
-                                e + 1 == D ? lse[i] : x[i][k + 1] * inv[i], through);
-          }
-        } else {
-#pragma unroll
-          for (int k = 0; k < NV; ++k) {
-            const int e = lane + 64 * k;
-            if (e < D) store_partial1(a.out, row + e, a.mid_dtype, x[i][k] * inv[i], through);
+        for (int k = 0; k < NW; ++k) {
+          const int w = lane + 64 * k;
+          if (first) {   // values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
+            const uint32_t next = w == D / 2 - 1 ? lse16[i] : hi[i][k];
+            store_bits32(row + 2 * w + 1, (lo[i][k] >> 16) | (next << 16), through);
+          } else {
+            store_bits32(row + 2 * w, lo[i][k], through);
           }
         }
       }
     }
     return;
   }
-  const int d = (lane % D4) * 4;
+  if (lane < nheads) {
+    const bool first_l = ((par0 + (uint64_t)hl * (uint64_t)a.so_h) & 1) != 0;
+    uint16_t* row = out + row0 + (int64_t)hl * a.so_h;
+    store_bits16(row + (first_l ? 0 : D), first_l ? (empty ? 0u : (uint32_t)r16[hl * D]) : lse16_l, through);
+  }
+  for (int h0 = 0; h0 < nheads; h0 += 4) {
+    uint32_t lo[4][NW], hi[4][NW], lse16[4];
+    int first[4];
 #pragma unroll
-  for (int r = 0; r < HB / RPI; ++r) {
-    const int h = r * RPI + lane / D4;
-    if (h >= nheads) continue;
-    f32x4 o = {0.f, 0.f, 0.f, 0.f};
-    float lse = -INFINITY;
-    if (!empty) {
-      const float M = part[HB * D + h];
-      const float L = part[HB * D + HB + h];
-      const float inv = L > 0.f ? 1.0f / L : 0.f;
-      o = *(const f32x4*)(part + h * D + d) * inv;
-      lse = L > 0.f ? (M + fd_log2(L)) * FD_LN2 : -INFINITY;
+    for (int i = 0; i < 4; ++i) {
+      const int hh = min(h0 + i, nheads - 1);
+      first[i] = (int)((par0 + (uint64_t)hh * (uint64_t)a.so_h) & 1);
+      lse16[i] = (uint32_t)__shfl((int)lse16_l, hh);
+#pragma unroll
+      for (int k = 0; k < NW; ++k) {
+        const int w = lane + 64 * k;   // dword of the parked row: values 2 w, 2 w + 1
+        lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
+        hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
+      }
     }
-    const int head = head0 + h;
-    const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
-    if (a.vec_out) {
-      store_partial4(a.out, off, a.mid_dtype, o, a.store_through != 0);
-    } else {
-      for (int i = 0; i < 4; ++i) store_from_f32(a.out, off + i, a.mid_dtype, o[i]);
-    }
-    if (d == 0 && !a.no_lse) {
-      if (a.lse) {
-        a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
-      } else {
-        store_from_f32(a.out, off + D, a.mid_dtype, lse);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (h0 + i >= nheads) break;
+      uint16_t* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
+#pragma unroll
+      for (int k = 0; k < NW; ++k) {
+        const int w = lane + 64 * k;
+        // a row that starts between two boundaries: values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
+        const uint32_t next = w == D / 2 - 1 ? lse16[i] : (hi[i][k] & 0xffffu);
+        const uint32_t word = first[i] ? (lo[i][k] >> 16) | (next << 16) : lo[i][k];
+        store_bits32(row + 2 * w + first[i], word, through);
       }
     }
   }

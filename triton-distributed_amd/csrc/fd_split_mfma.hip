@@ -44,6 +44,7 @@ constexpr int kKTile = kTile * kKRow;   // 8704 B of staged K per wave
 // LDS per wave: the K staging buffer, reused for the wave's partial result (16*NB heads x (128 + 2) floats)
 constexpr int wave_lds(int nb) { return nb == 1 ? kKTile : (16 * nb * kD + 2 * 16 * nb) * 4; }
 static_assert(wave_lds(1) >= (16 * kD + 2 * 16) * 4 && wave_lds(2) >= kKTile, "partial result and K tile share the buffer");
+static_assert(wave_lds(1) >= 16 * 4 + 16 * kD * 4 && wave_lds(2) >= 32 * 4 + 32 * kD * 4, "a finished fp32 partial fits the staging buffer");
 
 #ifndef FD_MFMA_OCC
 #define FD_MFMA_OCC
@@ -268,7 +269,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
     }
   };
   const int nheads = min(kHB, a.G - w.hb * kHB);
-  // Chunked work items: a finished split -> a parked slot as the finished partial (SplitArgs::park_final): fp32 LSEs,
+  // Chunked work items: a finished split -> a parked slot as the finished partial: fp32 LSEs of the head slots,
   // then normalised rows in mid_dtype.  A lane holds eight consecutive dims of head 16*nb + c per i.
   auto park_final = [&](char* slot) {
     wave_lds_fence();
@@ -333,11 +334,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       while (!(cur.end >= run_end && cur.base + kTile >= cur.end)) {   // all tiles but the wave's last one
         tile(cur.base, cur.end, lookup2, std::true_type{});
         if (cur.base + kTile >= cur.end) {   // that was the last tile of a split
-          if (a.park_final) {
-            park_final(park + parked * a.park_bytes);
-          } else {
-            stage_partial((float*)(park + parked * a.park_bytes));
-          }
+          park_final(park + parked * a.park_bytes);
           ++parked;
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
@@ -351,18 +348,13 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
         look = advance(look);
       }
       tile(cur.base, cur.end, lookup2, std::false_type{});
-      stage_partial(part);
+      park_final(kb);   // the wave's last split: its staging buffer is free now
       last_staged = true;
     }
     wave_lds_fence();
     for (int i = 0; s_cur + i < s_lim; ++i) {   // splits beyond the sequence's end are stored as empty
       const bool empty = i > parked || (i == parked && !last_staged);
-      if (i < parked && a.park_final) {
-        wave_copy_parked<kHB, kD>(a, park + i * a.park_bytes, w.b, head0, nheads, s_cur + i);
-      } else {
-        wave_store_partial<kHB, kD>(a, i < parked ? (const float*)(park + i * a.park_bytes) : part, w.b, head0, nheads,
-                                    s_cur + i, empty);
-      }
+      wave_copy_parked<kHB, kD>(a, i < parked ? park + i * a.park_bytes : kb, w.b, head0, nheads, s_cur + i, empty);
     }
   } else {
     if (t0 < t1) {
