@@ -187,7 +187,7 @@ def measure_target(torch, fd, dev, wl_cpu, steps, warmup, pools_n, ramp_ms, resi
     return round(us, 3), round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
 
 
-def _binding_step(torch, fd, dev):
+def _binding_step(torch, fd, dev, caller_partials):
     """The decode step through ``reference_binding.gqa_fwd_batch_decode`` (positional reference signature)."""
     import importlib.util
     path = os.path.join(os.path.dirname(os.path.abspath(fd.__file__)), "reference_binding.py")
@@ -202,10 +202,19 @@ def _binding_step(torch, fd, dev):
         out = torch.empty(B, Hq, D, dtype=wl.q.dtype, device=dev)
         q_lens = [1] * B
 
+        need = rb._lib.fd_workspace_bytes(__import__("ctypes").byref(rb.FdParams(
+            Hq, wl.k_cache.shape[2], D, wl.k_cache.shape[1], S, wl.k_cache.shape[0], wl.block_table.shape[1],
+            rb._DT[wl.q.dtype], rb._DT[wl.k_cache.dtype], 0, rb._DT[out.dtype])), B, 0, 0)
+        workspace = torch.empty(max(int(need), 256), dtype=torch.uint8, device=dev)
+
         def step(i):
             k, v = pools[i % len(pools)]
-            return rb.gqa_fwd_batch_decode(wl.q, k, v, None, q_lens, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap,
-                                           out_split, out, S)
+            if caller_partials:   # as the perf scripts and the sequence-parallel layer call it (test_decode_attn.py:322-331)
+                return rb.gqa_fwd_batch_decode(wl.q, k, v, None, q_lens, wl.kv_lens, wl.block_table, wl.scale,
+                                               wl.soft_cap, out_split, out, S)
+            # as the reference's tests call it (test_decode_attn.py:158): no output_split, the library plans
+            return rb.gqa_fwd_batch_decode(wl.q, k, v, workspace, q_lens, wl.kv_lens, wl.block_table, wl.scale,
+                                           wl.soft_cap, None, out, S)
         return step
     return factory
 
@@ -258,10 +267,14 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
                                                   resident=c2_resident, caller_partials=torch.float32))
     put("c2_caller_partials_bf16", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
                                                   resident=c2_resident, caller_partials=torch.bfloat16))
-    # ... and through the stand-alone ctypes binding a maintainer of the reference tree would add (fp32 partials of
-    # its own, no plan, nothing of this package's Python between the call and the library)
+    # ... and through the stand-alone ctypes binding a maintainer of the reference tree would add (nothing of this
+    # package's Python between the call and the library): without output_split, as the reference's tests call it --
+    # the library plans the step -- and with fp32 partials of the caller's own, as its perf scripts do
     put("c2_reference_binding", measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0,
-                                               resident=c2_resident, step_factory=_binding_step(torch, fd, dev)))
+                                               resident=c2_resident, step_factory=_binding_step(torch, fd, dev, False)))
+    put("c2_reference_binding_caller_partials",
+        measure_target(torch, fd, dev, U.make_config(2), steps, warmup, 4, 100.0, resident=c2_resident,
+                       step_factory=_binding_step(torch, fd, dev, True)))
     c5, c5t = U.make_config(5), U.make_config5_bf16_twin()
     put("c5_caller_partials_bf16", measure_target(torch, fd, dev, c5, steps, warmup, 4, 100.0,
                                                   caller_partials=torch.bfloat16))
@@ -462,6 +475,30 @@ def main():
     ms_per_step = max(gpu_ms, 0.0) / args.steps
     us_per_step = ms_per_step * 1e3
 
+    # ---- the same step as a prepared object (arguments marshalled once, one library call per step): what a serving
+    # loop that keeps its buffers would call; GPU time per step and the host's time to enqueue one
+    prepared_us = prepared_issue_us = None
+    if args.variant in ("plain", "persistent") and not args.exact_splits and not args.fuse and caller_dt is None:
+        kw_p = dict(variant=args.variant, output_combine=out, kv_split=S, lse_out=lse, path=args.path,
+                    waves_per_block=args.waves, workspace=workspace)
+        if wl.k_scale is not None:
+            kw_p.update(k_scale=wl.k_scale, v_scale=wl.v_scale)
+        if wl.extra_out is not None:
+            kw_p.update(extra_partials=(wl.extra_out, wl.extra_lse))
+        prepared = fd.PreparedDecode(wl.q, wl.k_cache, wl.v_cache, wl.kv_lens, wl.block_table, wl.scale, wl.soft_cap,
+                                     **kw_p)
+
+        def prepared_step(i):
+            k, v = pools[i % len(pools)]
+            return prepared(k_cache=k, v_cache=v)
+        prepared_us = _time_us(torch, prepared_step, args.steps, args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            prepared_step(i)
+        prepared_issue_us = (time.perf_counter() - t0) * 1e6 / args.steps
+        torch.cuda.synchronize()
+
     # ---- the same step replayed from a HIP graph (a serving loop captures its step): 8 steps per graph, rotating
     # over the pools like the eager loop
     graph_us = None
@@ -596,6 +633,8 @@ def main():
         # above ends after it and so can never be below the GPU's time per step)
         "host_issue_us_per_step": round(issue_us, 3),
         "hip_graph_replay_us_per_step": None if graph_us is None else round(graph_us, 3),
+        "prepared_step_us": None if prepared_us is None else round(prepared_us, 3),
+        "prepared_step_host_issue_us": None if prepared_issue_us is None else round(prepared_issue_us, 3),
         "clock_ramp_ms": round(ramp_ms),
         "timing": "HIP events around exactly `steps` back-to-back steps; 1 untimed lead-in step between the "
                   "synchronize and the first event keeps the host's first-launch latency out of the region",

@@ -1048,3 +1048,69 @@ def test_direct_output_c_abi_rules(fd):
     ref, ref_lse = oracle_decode(wl.to("cpu"))
     assert_out_close(out.cpu(), ref)
     assert_lse_close(lse.cpu(), ref_lse)
+
+
+def test_prepared_decode_step(fd):
+    """PreparedDecode: arguments marshalled once, launched many times -- the same bits as the wrappers, with new
+    contents in the same buffers, with rebound pools of the same geometry, and replayed from a HIP graph."""
+    wl = fd.utils.make_paged_workload("prepared", [1320, 18, 463, 2049, 0, 777], 32, 8, 128, 16, torch.bfloat16, 32, seed=71)
+    g = wl.to(DEV)
+    B, Hq, D = g.q.shape
+    ref, ref_lse = oracle_decode(wl)
+    for variant, fn in (("plain", fd.gqa_fwd_batch_decode), ("intra_rank", fd.gqa_fwd_batch_decode_intra_rank),
+                        ("persistent", fd.gqa_fwd_batch_decode_persistent)):
+        lse = torch.zeros(B, Hq, dtype=torch.float32, device=DEV)
+        kw = {} if variant == "intra_rank" else {"lse_out": lse}
+        step = fd.PreparedDecode(g.q, g.k_cache, g.v_cache, g.kv_lens, g.block_table, g.scale, variant=variant,
+                                 kv_split=g.kv_split, **kw)
+        out = step()
+        torch.cuda.synchronize()
+        want = fn(g.q, g.k_cache, g.v_cache, None, [1] * B, g.kv_lens, g.block_table, g.scale, kv_split=g.kv_split)
+        torch.cuda.synchronize()
+        assert out is step.output and torch.equal(out.view(torch.int16), want.view(torch.int16)), variant
+        assert_out_close(out[..., :D].cpu(), ref)
+        if variant != "intra_rank":
+            assert_lse_close(lse.cpu(), ref_lse)
+    # new contents in the same buffers, then other pools of the same geometry
+    lse = torch.zeros(B, Hq, dtype=torch.float32, device=DEV)
+    q, kc, vc, lens = g.q.clone(), g.k_cache.clone(), g.v_cache.clone(), g.kv_lens.clone()
+    step = fd.PreparedDecode(q, kc, vc, lens, g.block_table, g.scale, kv_split=-1, lse_out=lse)
+    import dataclasses
+    gen = torch.Generator().manual_seed(72)
+    wl2 = dataclasses.replace(
+        wl, q=torch.randn(wl.q.shape, generator=gen).to(torch.bfloat16),
+        k_cache=torch.randn(wl.k_cache.shape, generator=gen).to(torch.bfloat16),
+        v_cache=torch.randn(wl.v_cache.shape, generator=gen).to(torch.bfloat16),
+        block_table=torch.randint(0, wl.k_cache.shape[0], wl.block_table.shape, generator=gen, dtype=torch.int32),
+        kv_lens=torch.tensor([5, 2049, 1000, 64, 333, 0], dtype=torch.int32))
+    g2 = wl2.to(DEV)
+    q.copy_(g2.q)
+    lens.copy_(g2.kv_lens)
+    out = step(k_cache=g2.k_cache, v_cache=g2.v_cache, block_table=g2.block_table)
+    torch.cuda.synchronize()
+    ref2, ref2_lse = oracle_decode(wl2)
+    assert_out_close(out.cpu(), ref2)
+    assert_lse_close(lse.cpu(), ref2_lse)
+    with pytest.raises(RuntimeError, match="must keep shape"):
+        step(k_cache=g2.k_cache[:-1])
+    with pytest.raises(RuntimeError, match="planned step"):
+        fd.PreparedDecode(q, kc, vc, lens, g.block_table, g.scale, fuse_combine=True)
+    # in a HIP graph: replays follow the contents of the buffers
+    step = fd.PreparedDecode(q, g2.k_cache, g2.v_cache, lens, g2.block_table, g.scale, lse_out=lse)
+    step()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    torch.cuda.synchronize()
+    for new_lens in ([5, 2049, 1000, 64, 333, 0], [2049, 1, 0, 700, 2049, 31]):
+        lens.copy_(torch.tensor(new_lens, dtype=torch.int32))
+        step.output.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        wl2.kv_lens = torch.tensor(new_lens, dtype=torch.int32)
+        r3, r3_lse = oracle_decode(wl2)
+        assert_out_close(step.output.cpu(), r3)
+        assert_lse_close(lse.cpu(), r3_lse)

@@ -221,6 +221,11 @@ def test_split_plan_policy(fd):
     assert plan(1, 96, 12, 32, 65536, P=1) == 32   # the caller's bound wins
     assert plan(1, 8, 1, 256, 65536) == 256        # one KV head: one split per CU
     assert plan(1, 96, 12, 128, 1 << 20, P=1) == 42
+    # short tables with 12 and 24 (KV head, head block) groups keep that rule: one- and two-tile splits were measured
+    # level with or ahead of fewer, longer ones (3 x 512 tokens: 7.5 us with 10 splits, 8.4 / 9.3 us with 4 / 2)
+    assert plan(3, 32, 8, 32, 32) == 10 and plan(3, 32, 8, 32, 64) == 10       # 512- and 1024-token tables, 24 groups
+    assert plan(1, 96, 12, 32, 2048, P=1) == 21 and plan(1, 96, 12, 32, 512, P=1) == 21   # 12 groups
+    assert plan(2, 96, 12, 32, 1024, P=1) == 10                                 # 24 groups of one head
     assert plan(1, 8, 8, 1, 4) == 1                # never below 1, never above what the caller asked for
     assert plan(4096, 32, 8, 32, 1) == 1
     # the part of the plan that fills the chip, without the bound on the length of a split: what a sequence gets

@@ -103,6 +103,7 @@ constexpr int64_t kTargetWavesValu = 2048;
 constexpr int64_t kMinWorkgroups = 256;
 constexpr int64_t kMaxTokensPerSplit = kMaxTokensPerRange;   // keeps a ragged batch balanceable by the dispatcher
 constexpr int64_t kMaxBalanceSplits = 32;                    // ... with at most this many splits for that purpose
+constexpr int kPlanMinTokensPerSplit = 0;                    // fewest tokens a planned split of a full-length sequence holds
 constexpr int64_t kStoreThroughBytes = 16 << 20;   // partials of a step from which on they are written through
 constexpr int kMaxChunkBatch = 32;     // chunked work items: largest batch they are used for
 constexpr int kMaxSplitsPerWave = 4;   // chunked work items: splits one wave walks (finished partials parked in LDS)
@@ -720,6 +721,23 @@ int fd_plan_splits(const fd_params* p, int32_t batch) {
   // mostly empty workgroups in front of the chip); sequences beyond 32 x 4096 tokens get longer ranges instead.
   if (batch > 1) {
     while (s * kMaxTokensPerSplit < max_tokens && s < kMaxBalanceSplits) s <<= 1;
+  }
+  // No floor on the tokens of a split by default: cutting a short table into one- and two-tile splits was measured
+  // against fewer, longer ones (FD_PLAN_MIN_TOKENS = 64 ... 512; graph replays) and the many short splits are level or
+  // ahead -- 3 sequences of 512 tokens on 8 KV heads 7.5 us with 10 splits against 8.4 / 9.3 us with 4 / 2, of 1024
+  // tokens 7.8 against 8.5 / 9.3 / 10.5 us with 8 / 4 / 2, one query on 12 KV heads over 2048 tokens 9.0 us with 21
+  // splits against 9.9 / 12.2 us with 8 / 4: such steps are latency, and more workgroups hide more of it.
+  {
+    static const int min_tokens = env_int("FD_PLAN_MIN_TOKENS") > 0 ? env_int("FD_PLAN_MIN_TOKENS") : kPlanMinTokensPerSplit;
+    if (min_tokens > 0) {
+      int64_t most = max_tokens / min_tokens;
+      if (most < 1) most = 1;
+      if (s > most) {
+        const bool was_pow2 = (s & (s - 1)) == 0;
+        s = most;
+        if (was_pow2) while (s & (s - 1)) s &= s - 1;   // stay a power of two
+      }
+    }
   }
   // Powers of two where the shape allows: with sequence lengths that are powers of two (or multiples of large ones)
   // every split then starts on a tile boundary and the waves of a workgroup get equal runs.

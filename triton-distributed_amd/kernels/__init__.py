@@ -10,6 +10,9 @@ from .flash_decode import (  # noqa: F401
     kernel_inter_rank_gqa_fwd_batch_decode_combine_kv,
     inter_rank_combine,
     schedule_sequences,
+    PreparedDecode,
+    decode_plan,
+    workspace_bytes,
     get_split_kv_algo_info,
     get_combine_kv_algo_info,
     get_triton_split_kv_algo_info,
@@ -40,4 +43,7 @@ __all__ = [
     "kernel_inter_rank_gqa_fwd_batch_decode_combine_kv",
     "inter_rank_combine",
     "schedule_sequences",
+    "PreparedDecode",
+    "decode_plan",
+    "workspace_bytes",
 ]

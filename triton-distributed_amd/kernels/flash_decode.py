@@ -233,7 +233,8 @@ _STEP_CACHE = {}   # fd_decode_args images of planned steps by everything but th
 def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, output_split, output_combine,
             kv_split, *, with_lse_column: bool, lse_out=None, k_scale=None, v_scale=None, extra_partials=None, seq_order=None,
             seq_order_lens=None, stream=None, path="auto", waves_per_block=0, fuse_combine=False, plan_splits=True,
-            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False, auto_order=True, rank_merge=None):
+            schedule_items=False, item_order=None, max_kv_len=None, no_alloc=False, auto_order=True, rank_merge=None,
+            _prepare=False):
     batch, q_heads, q_head_dim = q.shape
     _, page_size, kv_heads, k_head_dim = k_cache.shape
     v_shape = v_cache.shape
@@ -345,11 +346,15 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
             a.params.k_scale, a.params.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
         if rm is not None:
             a.params.rank_merge = addressof(rm)
+        if _prepare:   # PreparedDecode: the marshalled step and what must stay alive with it
+            return a, (hold, rm, output_combine)
         rc = lib.fd_decode_planned(hstream, byref(a))
         if rc:
             check(rc)
         return output_combine
 
+    if _prepare:
+        raise RuntimeError("PreparedDecode covers the planned step: no output_split, fuse_combine or no_alloc")
     # ---- explicit calls: the caller's own partial buffer (exactly kv_split splits with the reference's ranges, layout
     # [B, Hq, S, Dv + 1]), the fused single launch, or partials in the library's static array.  How the step is issued
     # still comes from the library's plan.
@@ -440,6 +445,67 @@ def _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_ca
         ex_out.data_ptr() if n_extra else None, ex_lse.data_ptr() if n_extra else None, n_extra,
         tickets.data_ptr() if tickets is not None else None, byref(p)))
     return output_combine
+
+
+class PreparedDecode:
+    """A planned decode step whose arguments are marshalled once (``fd_decode_args``) and launched many times: a
+    serving loop decodes with the same buffers step after step -- the query buffer, the cache pools, the block table,
+    ``kv_lens`` and the output keep their addresses, only their contents change -- so all that is left per step is one
+    library call (about 6 us on the host with its two launches, against about 10 us through the wrappers, which check
+    and marshal two dozen arguments every time, as the reference's do, flash_decode.py:788-844).
+
+        step = PreparedDecode(q, k_cache, v_cache, kv_lens, block_table, scale, output_combine=out, lse_out=lse)
+        for _ in range(n):
+            ...                       # new contents in q / the caches / kv_lens / block_table
+            step()                    # -> out
+
+    ``variant``: "plain" (``gqa_fwd_batch_decode``), "intra_rank" (merged LSE in the output's last column) or
+    "persistent" (the scheduled variant).  Every keyword of the planned step is accepted (``kv_split``, ``soft_cap``,
+    ``k_scale`` / ``v_scale``, ``extra_partials``, ``seq_order``, ``max_kv_len``, ``workspace`` ...).  The object keeps
+    the tensors alive; ``step(k_cache=..., v_cache=...)`` rebinds tensors of the same shape, dtype and strides (a
+    rotating pool).  Calls on one object must not overlap: they share its workspace.  Capturable into a HIP graph
+    like the wrappers (the step allocates nothing)."""
+
+    _REBINDABLE = {"q": "q", "k_cache": "k_cache", "v_cache": "v_cache", "kv_lens": "kv_lens",
+                   "block_table": "block_table", "output_combine": "out", "lse_out": "lse_out"}
+
+    def __init__(self, q, k_cache, v_cache, kv_lens, block_table, scale, soft_cap=0.0, *, variant="plain",
+                 output_combine=None, kv_split=-1, workspace=None, stream=None, **kw):
+        if variant not in ("plain", "intra_rank", "persistent"):
+            raise ValueError(f"variant {variant!r}")
+        if variant == "persistent" and kw.get("seq_order") is None and kw.get("item_order") is None and q.shape[0] > 1:
+            kw["schedule_items"] = True
+        cols = v_cache.shape[-1] + (1 if variant == "intra_rank" else 0)
+        if output_combine is None:
+            output_combine = torch.empty(q.shape[0], q.shape[1], cols, dtype=q.dtype, device=q.device)
+        self._lib = load_library()
+        self._stream = stream
+        self._device = q.device.index
+        self._args, self._keep = _decode(q, k_cache, v_cache, workspace, kv_lens, block_table, scale, soft_cap, None,
+                                         output_combine, kv_split, with_lse_column=variant == "intra_rank",
+                                         stream=stream, _prepare=True, **kw)
+        self._ref = byref(self._args)
+        self._tensors = dict(q=q, k_cache=k_cache, v_cache=v_cache, kv_lens=kv_lens, block_table=block_table,
+                             output_combine=output_combine, lse_out=kw.get("lse_out"), kw=kw)
+        self.output = output_combine
+
+    def __call__(self, stream=None, **rebind):
+        for name, t in rebind.items():
+            field = self._REBINDABLE[name]
+            old = self._tensors[name]
+            if old is None or t.shape != old.shape or t.stride() != old.stride() or t.dtype != old.dtype \
+                    or t.device != old.device:
+                raise RuntimeError(f"PreparedDecode: {name} must keep shape, strides, dtype and device")
+            setattr(self._args, field, t.data_ptr())
+            self._tensors[name] = t
+            if name == "output_combine":
+                self.output = t
+        s = stream if stream is not None else self._stream
+        rc = self._lib.fd_decode_planned(s.cuda_stream if s is not None else stream_handle(None, self._device),
+                                         self._ref)
+        if rc:
+            check(rc)
+        return self.output
 
 
 _PLAN_CACHE = {}   # fd_plan_decode results by problem shape
