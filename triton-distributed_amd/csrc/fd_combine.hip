@@ -219,20 +219,27 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_kernel(const Combi
 // latency.  Thread (r, c): partials r, r + ROWS, ... and 128-bit column chunk c.  Lane i of every wave loads LSE i
 // (MAXP <= 64 = one per lane); the maximum is a butterfly over the wave and a thread takes the LSEs of its own
 // partials from the lanes that hold them, so nothing goes through LDS before the final sum.
-template <int D, int MAXP, int MID, bool VEC>
+template <int D, int MAXP, int MID, bool VEC, int CG>
 __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const CombineArgs a) {
-  constexpr int CG = D / 4;
+  // CG column groups of four columns per workgroup: D / 4 = the whole output row (one workgroup per row), or fewer --
+  // D / 4 / CG workgroups per row -- where a step has few output rows and many partials (one long sequence), so that
+  // the chip sees at least a workgroup per CU and a thread walks few partials.
   constexpr int ROWS = kCombineThreads / CG;
   constexpr int PASSES = (MAXP + ROWS - 1) / ROWS;
+  constexpr int CHUNKS = D / 4 / CG;
+  constexpr int NCOL = 4 * CG;
   static_assert(MAXP <= 64, "one LSE per lane");
-  __shared__ __align__(16) float s_acc[ROWS][D];
+  static_assert(VEC || CG == D / 4, "column-strided rows come as whole rows");
+  __shared__ __align__(16) float s_acc[ROWS][NCOL];
   __shared__ float s_l[ROWS];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int b = blockIdx.x / a.Hq;
-  const int h = blockIdx.x - b * a.Hq;
+  const int row = CHUNKS == 1 ? (int)blockIdx.x : (int)blockIdx.x / CHUNKS;
+  const int col0 = CHUNKS == 1 ? 0 : ((int)blockIdx.x - row * CHUNKS) * NCOL;
+  const int b = row / a.Hq;
+  const int h = row - b * a.Hq;
   const int S = a.num_partials;
-  const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh;
+  const int64_t mid_base = (int64_t)b * a.s_mb + (int64_t)h * a.s_mh + col0;
   const int r = tid / CG;
   const int c = tid - r * CG;
   // VEC: rows start on multiples of four elements and a thread owns columns 4c .. 4c + 3 (one 128- or 64-bit load);
@@ -265,7 +272,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
   float mine = -INFINITY;   // LSE of partial `lane`: from its own buffer, or from column D of the partial's row
   if (lane < S) {
     mine = a.mid_lse ? a.mid_lse[((int64_t)b * a.Hq + h) * S + lane]
-                     : load_as_f32(a.mid_o, mid_base + (int64_t)lane * a.s_ms + D, MID);
+                     : load_as_f32(a.mid_o, mid_base - col0 + (int64_t)lane * a.s_ms + D, MID);
     // partials of other ranks: rank `lane` counts iff it holds tokens of this sequence (flash_decode.py:513-515);
     // what its slot holds otherwise is not looked at (the rows are requested, their values dropped below)
     if (a.mode == FD_COMBINE_RANK && a.seqlens[(int64_t)lane * a.batch + b] <= 0) mine = -INFINITY;
@@ -291,7 +298,7 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
   }
   if (c == 0) s_l[r] = L;
   __syncthreads();
-  if (tid < D) {
+  if (tid < NCOL) {
     float v = 0.f, Lsum = 0.f;
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
@@ -300,8 +307,8 @@ __global__ void __launch_bounds__(kCombineThreads) fd_combine_own_kernel(const C
     }
     const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
     const int64_t out_base = (int64_t)b * a.s_ob + (int64_t)h * a.s_oh;
-    store_from_f32(a.out, out_base + tid, a.out_dtype, v * inv);
-    if (tid == 0) {
+    store_from_f32(a.out, out_base + col0 + tid, a.out_dtype, v * inv);
+    if (tid == 0 && col0 == 0) {
       const float res = Lsum > 0.f ? M + __logf(Lsum) : -INFINITY;
       if (a.mode == FD_COMBINE_SPLIT_LSE) store_from_f32(a.out, out_base + D, a.out_dtype, res);
       if (a.lse_out) a.lse_out[(int64_t)b * a.Hq + h] = res;
@@ -339,33 +346,36 @@ int fd_launch_combine(hipStream_t stream, const CombineArgs& args) {
   CombineArgs a = args;
   const int64_t rows = (int64_t)a.batch * a.Hq;
   void (*kern)(const CombineArgs) = nullptr;
-  // the short kernel: this library's own partials in the same call (all slots written) or the per-rank partials of the
-  // inter-rank merge (validity by the ranks' lengths), at most 64 of them -- above
-  // 32 only where there is a workgroup per CU: with few output rows (one long sequence: 96 rows x 42 partials) the
-  // general kernel, which spreads a row over several workgroups, is the faster one (5.0 against 5.7 us)
+  // The short kernel: this library's own partials in the same call (all slots written) or the per-rank partials of the
+  // inter-rank merge (validity by the ranks' lengths), at most 64 of them and no extras.  Rows that are readable four
+  // values at a time are spread over several workgroups where the step has few output rows (one long sequence: 96
+  // rows x 42 partials as 384 workgroups of 32 columns: 4.5 -> 3.1 us behind the split kernel against the general
+  // kernel's run-time loops); the caller's [.., D + 1] rows come as whole rows.
   const int np_own = a.num_partials <= 16 ? 16 : (a.num_partials <= 32 ? 32 : 64);
   const bool small = (a.all_slots_written || a.mode == FD_COMBINE_RANK) && a.num_extra == 0 && !a.local_out &&
-                     (a.num_partials <= 32 || (a.num_partials <= 64 && rows >= 256));
-  // General kernel: column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under
-  // one workgroup per CU and a thread would still have more than two partials to walk.
+                     a.num_partials <= 64 && (a.vec_mid || a.num_partials <= 32 || rows >= 256);
+  // Column groups per workgroup.  Start with the whole row (D/4) and halve while the grid is under one workgroup per
+  // CU and a thread would still have more than two partials to walk (short kernel: down to 8 groups of four columns).
   int cg = a.D / 4;
   const int64_t np = (int64_t)a.num_partials + a.num_extra;
-  while (!small && cg > 4 && rows * (a.D / 4 / cg) < 256 && np > 2 * (kCombineThreads / cg)) cg >>= 1;
+  const int cg_min = small ? 8 : 4;
+  while ((!small || a.vec_mid) && cg > cg_min && rows * (a.D / 4 / cg) < 256 && np > 2 * (kCombineThreads / cg)) cg >>= 1;
   a.cg_shift = 0;
   while ((1 << a.cg_shift) < cg) ++a.cg_shift;
-  const int64_t wgs = small ? rows : rows * (a.D / 4 / cg);
+  const int64_t wgs = rows * (a.D / 4 / cg);
   if (wgs >= ((int64_t)1 << 31)) return FD_ERR_TOO_LARGE;
   const unsigned grid = (unsigned)wgs;
-#define FD_OWN_V(D_, M_, V_) (np_own == 16 ? fd_combine_own_kernel<D_, 16, M_, V_> : np_own == 32 ? fd_combine_own_kernel<D_, 32, M_, V_> : fd_combine_own_kernel<D_, 64, M_, V_>)
-#define FD_OWN_P(D_, M_) (a.vec_mid ? FD_OWN_V(D_, M_, true) : FD_OWN_V(D_, M_, false))
-#define FD_OWN(D_) (a.mid_dtype == FD_F32 ? FD_OWN_P(D_, FD_F32) : a.mid_dtype == FD_F16 ? FD_OWN_P(D_, FD_F16) : FD_OWN_P(D_, FD_BF16))
+#define FD_OWN_N(D_, M_, V_, C_) (np_own == 16 ? fd_combine_own_kernel<D_, 16, M_, V_, C_> : np_own == 32 ? fd_combine_own_kernel<D_, 32, M_, V_, C_> : fd_combine_own_kernel<D_, 64, M_, V_, C_>)
+#define FD_OWN_V(D_, M_) (!a.vec_mid ? FD_OWN_N(D_, M_, false, D_ / 4) : cg == D_ / 4 ? FD_OWN_N(D_, M_, true, D_ / 4) : \
+                          cg == D_ / 8 ? FD_OWN_N(D_, M_, true, (D_ / 8 >= 8 ? D_ / 8 : 8)) : cg == 16 ? FD_OWN_N(D_, M_, true, 16) : FD_OWN_N(D_, M_, true, 8))
+#define FD_OWN(D_) (a.mid_dtype == FD_F32 ? FD_OWN_V(D_, FD_F32) : a.mid_dtype == FD_F16 ? FD_OWN_V(D_, FD_F16) : FD_OWN_V(D_, FD_BF16))
   switch (a.D) {
     case 64: kern = small ? FD_OWN(64) : fd_combine_kernel<64>; break;
     case 128: kern = small ? FD_OWN(128) : fd_combine_kernel<128>; break;
     case 256: kern = small ? FD_OWN(256) : fd_combine_kernel<256>; break;
     default: return FD_ERR_UNSUPPORTED;
   }
-#undef FD_OWN_P
+#undef FD_OWN_N
 #undef FD_OWN_V
 #undef FD_OWN
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kCombineThreads), 0, stream, a);
