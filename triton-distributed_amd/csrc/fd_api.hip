@@ -402,7 +402,10 @@ int split_impl(const char* fn, void* stream, const void* q, const void* k_cache,
   // Chunked work items: the caller's split count and ranges are kept exactly (they are observable in out_split), but a
   // workgroup walks `chunk` consecutive splits, so that the chip sees about as many work items as the library's own
   // plan would launch: every work item pays the prologue (arguments -> length -> block table -> first rows) once, not
-  // once per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.
+  // once per split.  Kernels that have this form: head_dim 128, 16-bit and fp8 caches.  (The head_dim 64 and 256
+  // kernels were given it as well and measured level with one workgroup per split -- config 2's shape with 32
+  // caller-visible bf16 partials: head_dim 256 91.8 against 92.4 us, head_dim 64 27.9 against 27.3 us; in the
+  // library's own layout 90.4 against 89.7 and 26.6 against 26.2 us -- so they launch a workgroup per split.)
   // Not for large batches: their lengths differ in practice, and many short work items balance better over the CUs
   // than few long ones (config 4's ragged batch of 64 with exactly 32 splits: 691 us unchunked, 713 us chunked).
   ChunkPlan cp = chunk_plan(1, false);

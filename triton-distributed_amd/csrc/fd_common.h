@@ -826,7 +826,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
   const int lane = threadIdx.x & 63;
   constexpr int D4 = D / 4;
   constexpr int RPI = 64 / D4;
-  static_assert(D4 <= 64 && HB % RPI == 0 && D % 128 == 0, "one wave covers whole rows");
+  static_assert(D4 <= 64 && HB % RPI == 0 && D % 64 == 0, "one wave covers whole rows");
   const float* lse_slot = (const float*)slot;
   const char* rows = slot + HB * 4;
   const bool through = a.store_through != 0;
@@ -916,7 +916,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
   }
   // element parity of a row's start relative to a 4-byte boundary
   const uint64_t par0 = (reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row0;
-  constexpr int NW = D / 128;   // dwords per lane and row
+  constexpr int NW = (D / 2 + 63) / 64;   // dwords per lane and row (D = 64: half the lanes are idle)
   if ((a.so_h & 1) == 0) {
     // The usual case -- an even number of splits, so that all heads of a split start with the same parity: one
     // wave-uniform decision instead of one per row.
@@ -933,7 +933,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
         if (first) lse16[i] = f32_to_bits16(empty ? -INFINITY : lse_slot[hh], a.mid_dtype);
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
-          const int w = lane + 64 * k;   // dword of the parked row: values 2 w, 2 w + 1
+          const int w = min(lane + 64 * k, D / 2 - 1);   // dword of the parked row: values 2 w, 2 w + 1
           lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
           if (first) hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
         }
@@ -945,6 +945,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
           const int w = lane + 64 * k;
+          if (w >= D / 2) continue;
           if (first) {   // values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
             const uint32_t next = w == D / 2 - 1 ? lse16[i] : hi[i][k];
             store_bits32(row + 2 * w + 1, (lo[i][k] >> 16) | (next << 16), through);
@@ -971,7 +972,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
       lse16[i] = (uint32_t)__shfl((int)lse16_l, hh);
 #pragma unroll
       for (int k = 0; k < NW; ++k) {
-        const int w = lane + 64 * k;   // dword of the parked row: values 2 w, 2 w + 1
+        const int w = min(lane + 64 * k, D / 2 - 1);   // dword of the parked row: values 2 w, 2 w + 1
         lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
         hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
       }
@@ -983,6 +984,7 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
 #pragma unroll
       for (int k = 0; k < NW; ++k) {
         const int w = lane + 64 * k;
+        if (w >= D / 2) continue;
         // a row that starts between two boundaries: values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
         const uint32_t next = w == D / 2 - 1 ? lse16[i] : (hi[i][k] & 0xffffu);
         const uint32_t word = first[i] ? (lo[i][k] >> 16) | (next << 16) : lo[i][k];
