@@ -47,6 +47,10 @@ def parse_args():
     ap.add_argument("--caller-partials", default=None, choices=["fp32", "fp16", "bf16"],
                     help="the caller hands in output_split [B, Hq, S, D + 1] of this type, as the reference's perf "
                          "scripts and its sequence-parallel layer do: exactly kv_split observable partials")
+    ap.add_argument("--launch-decomposition", action="store_true",
+                    help="also time, as HIP-graph replays (no host in the loop): the split kernel alone, split + combine, "
+                         "split + a 64-element fill kernel, and that fill kernel alone -- what the second launch of a "
+                         "step costs whatever it computes")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-targets", action="store_true",
@@ -573,6 +577,58 @@ def main():
     split_us = e0.elapsed_time(e1) * 1e3 / args.steps
     achieved = algo_bytes / (split_us * 1e-6) / 1e9
 
+    # ---- what the second launch costs: graph replays of 20 launches each (best of 7 timings of 10 replays)
+    decomposition = None
+    if args.launch_decomposition:
+        tiny = torch.zeros(64, device=dev)
+
+        def graph_us(fn, n=20):
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                fn(0)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(n):
+                    fn(i)
+            for _ in range(20):
+                g.replay()
+            best = float("inf")
+            for _ in range(7):
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(10):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e3 / (10 * n))
+            return round(best, 3)
+
+        def split_graph(i):   # (the capture stream differs from the stream the leg above launched on)
+            k, v = pools[i % len(pools)]
+            fd._lib.check(lib.fd_split_kv(
+                torch.cuda.current_stream().cuda_stream, wl.q.data_ptr(), k.data_ptr(), v.data_ptr(), mid.data_ptr(),
+                lse_split_ptr, float(wl.scale), wl.block_table.data_ptr(), wl.kv_lens.data_ptr(), B,
+                wl.q.stride(0), wl.q.stride(1), k.stride(-3), k.stride(-2), v.stride(-3), v.stride(-2),
+                mid.stride(0), mid.stride(1), mid.stride(2), wl.block_table.stride(0), order_ptr, byref(p)))
+
+        def split_then_fill(i):
+            split_graph(i)
+            tiny.zero_()
+        decomposition = {
+            "method": "HIP-graph replays of 20 launches (or launch pairs), best of 7 timings of 10 replays, us per launch (pair)",
+            "split_kernel_us": graph_us(split_graph),
+            "split_plus_combine_us": graph_us(step),
+            "split_plus_64_element_fill_us": graph_us(split_then_fill),
+            "fill_kernel_alone_us": graph_us(lambda i: tiny.zero_()),
+        }
+        decomposition["second_launch_floor_us"] = round(
+            decomposition["split_plus_64_element_fill_us"] - decomposition["split_kernel_us"], 3)
+        decomposition["combine_work_beyond_the_floor_us"] = round(
+            decomposition["split_plus_combine_us"] - decomposition["split_plus_64_element_fill_us"], 3)
+
     if args.copy_ref:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
         dst = torch.empty_like(src)
@@ -628,6 +684,7 @@ def main():
         "hbm_gbps_step": round(algo_bytes / (us_per_step * 1e-6) / 1e9, 1),
         "hbm_pct_of_peak_step": round(100.0 * algo_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes": algo_bytes,
+        "library_build_id": lib.fd_build_id().decode(),
         "host_wall_ms_per_step": round(wall_ms / args.steps, 6),
         # the host's own share: wall time per step up to the last enqueue, before the synchronize (the wall figure
         # above ends after it and so can never be below the GPU's time per step)
@@ -665,6 +722,8 @@ def main():
     if headline and not args.no_targets:
         targets = measure_targets(torch, fd, dev, args.steps, args.warmup, (wl, pools))
 
+    if decomposition is not None:
+        result["launch_decomposition"] = decomposition
     if not args.no_write_side:
         result["write_side"] = measure_write_side(torch, fd, wl, dev, args.steps, args.warmup, step, pools, S)
         block = measure_decode_block(torch, fd, wl, dev, args.steps, args.warmup)
