@@ -582,7 +582,7 @@ def main():
     if args.launch_decomposition:
         tiny = torch.zeros(64, device=dev)
 
-        def graph_us(fn, n=20):
+        def replay_us(fn, n=20):
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -619,10 +619,10 @@ def main():
             tiny.zero_()
         decomposition = {
             "method": "HIP-graph replays of 20 launches (or launch pairs), best of 7 timings of 10 replays, us per launch (pair)",
-            "split_kernel_us": graph_us(split_graph),
-            "split_plus_combine_us": graph_us(step),
-            "split_plus_64_element_fill_us": graph_us(split_then_fill),
-            "fill_kernel_alone_us": graph_us(lambda i: tiny.zero_()),
+            "split_kernel_us": replay_us(split_graph),
+            "split_plus_combine_us": replay_us(step),
+            "split_plus_64_element_fill_us": replay_us(split_then_fill),
+            "fill_kernel_alone_us": replay_us(lambda i: tiny.zero_()),
         }
         decomposition["second_launch_floor_us"] = round(
             decomposition["split_plus_64_element_fill_us"] - decomposition["split_kernel_us"], 3)
