@@ -807,19 +807,26 @@ __device__ __forceinline__ uint32_t f32_to_bits16(float x, int dtype) {
                          : (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
 }
 
+// Vectors in global memory that are only known to start on a 4-byte boundary: global loads and stores of two or four
+// dwords need no more than dword alignment on this target.
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
 // Chunked work items: ONE wave copies a finished partial that it parked in LDS (HB fp32 LSEs, then the normalised
 // rows [head][D] of its real heads in mid_dtype) to split s of its head slots.  Called at the end of the wave's run
 // only: on this target stores and loads of a wave retire in order (one vmcnt), so a store issued between two tiles
 // would hold back every later K/V load until it is acknowledged.  empty: the split holds no token (out = 0,
-// lse = -inf; the slot is not read).
-//  * Rows that start on multiples of four elements (the library's own layout): four values per lane, whole rows per
-//    store instruction.
-//  * Else (the reference's [B, Hq, S, D + 1] layout, whose rows are D + 1 elements apart): consecutive lanes on
-//    consecutive elements, so that a store instruction still covers contiguous memory.  A 16-bit row of D values with
-//    the LSE behind them goes out as dwords of two values on 4-byte boundaries: a row that starts between two
-//    boundaries stores value 0 alone and pairs (1, 2) .. (D - 1, LSE); one that starts on a boundary pairs (0, 1) ..
-//    (D - 2, D - 1) and stores the LSE alone.  The values are the parked bits: nothing is scaled or converted here
-//    but the LSE, and every LDS read of four rows is requested before the first store.
+// lse = -inf; the slot is not read).  Every form moves 128 bits per lane (64 for 16-bit rows on multiples of four
+// elements) with whole rows per store instruction, and the values are the parked bits: nothing is scaled or
+// converted here but the LSE.
+//  * fp32 rows, and 16-bit rows that start on multiples of four elements (the library's own layout): straight copies.
+//    fp32 rows of the reference's [B, Hq, S, D + 1] layout start on 4-byte boundaries only, which is all a 128-bit
+//    store needs.
+//  * 16-bit rows of that layout (D values with the LSE behind them, D + 1 elements apart, so every other row starts
+//    between two 4-byte boundaries): a row that starts on a boundary goes out as it is parked and its LSE alone; one
+//    that starts between two stores value 0 alone and then the 128-bit pieces (1 .. 8), (9 .. 16), .. (D - 7 .. D - 1,
+//    LSE), each put together from five parked dwords with a funnel shift.  The LDS reads of all rows are independent
+//    of each other, so the wave pays one LDS round trip, not one per row.
 template <int HB, int D>
 __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char* slot, int b, int head0, int nheads,
                                                  int s, bool empty) {
@@ -830,7 +837,10 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
   const float* lse_slot = (const float*)slot;
   const char* rows = slot + HB * 4;
   const bool through = a.store_through != 0;
-  if (a.vec_out) {
+  constexpr int LPR = D / 8;      // 16-bit rows: lanes per row, eight values each
+  constexpr int RPS = 64 / LPR;   // ... and rows per store instruction
+  static_assert(HB % RPS == 0, "one wave covers whole rows");
+  if (a.mid_dtype == FD_F32) {
     const int d = (lane % D4) * 4;
 #pragma unroll
     for (int r = 0; r < HB / RPI; ++r) {
@@ -838,22 +848,38 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
       if (h >= nheads) continue;
       const int head = head0 + h;
       const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
-      if (a.mid_dtype == FD_F32) {
-        const f32x4 v = empty ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)((const float*)rows + h * D + d);
-        float* p = (float*)a.out + off;
-        if (through) {
-          asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-        } else {
-          *(f32x4*)p = v;
-        }
+      const f32x4 v = empty ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)((const float*)rows + h * D + d);
+      float* p = (float*)a.out + off;
+      if (through) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
       } else {
-        const u32x2 v = empty ? u32x2{0u, 0u} : *(const u32x2*)((const uint16_t*)rows + h * D + d);
-        uint16_t* p = (uint16_t*)a.out + off;
-        if (through) {
-          asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+        *(f32x4_a4*)p = v;
+      }
+      if (d == 0 && !a.no_lse) {
+        const float lse = empty ? -INFINITY : lse_slot[h];
+        if (a.lse) {
+          a.lse[((int64_t)b * a.Hq + head) * a.S + s] = lse;
         } else {
-          *(u32x2*)p = v;
+          store_partial1(a.out, off + D, a.mid_dtype, lse, through);
         }
+      }
+    }
+    return;
+  }
+  if (a.vec_out) {
+    const int d = (lane % LPR) * 8;
+#pragma unroll
+    for (int r = 0; r < HB / RPS; ++r) {
+      const int h = r * RPS + lane / LPR;
+      if (h >= nheads) continue;
+      const int head = head0 + h;
+      const int64_t off = (int64_t)b * a.so_b + (int64_t)head * a.so_h + (int64_t)s * a.so_s + d;
+      const u32x4 v = empty ? u32x4{0u, 0u, 0u, 0u} : *(const u32x4*)((const uint16_t*)rows + h * D + d);
+      uint16_t* p = (uint16_t*)a.out + off;
+      if (through) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+      } else {
+        *(u32x4_a4*)p = v;
       }
       if (d == 0 && !a.no_lse) {
         const float lse = empty ? -INFINITY : lse_slot[h];
@@ -867,41 +893,12 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
     return;
   }
   const int64_t row0 = (int64_t)b * a.so_b + (int64_t)head0 * a.so_h + (int64_t)s * a.so_s;
-  // lane h serves row h's single values: its LSE (and, for paired 16-bit rows, the row's odd value)
-  const int hl = lane < nheads ? lane : nheads - 1;
-  const float lse_l = empty ? -INFINITY : lse_slot[hl];
-  if (a.mid_dtype == FD_F32) {
-    constexpr int NV = D / 64;
-    float* out = (float*)a.out;
-    for (int h0 = 0; h0 < nheads; h0 += 4) {
-      uint32_t x[4][NV];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int hh = min(h0 + i, nheads - 1);
-#pragma unroll
-        for (int k = 0; k < NV; ++k) x[i][k] = empty ? 0u : ((const uint32_t*)rows)[hh * D + lane + 64 * k];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (h0 + i >= nheads) break;
-        float* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
-#pragma unroll
-        for (int k = 0; k < NV; ++k) store_bits32(row + lane + 64 * k, x[i][k], through);
-      }
-    }
-    if (lane < nheads && !a.no_lse) {
-      if (a.lse) {
-        a.lse[((int64_t)b * a.Hq + head0 + hl) * a.S + s] = lse_l;
-      } else {
-        store_bits32(out + row0 + (int64_t)hl * a.so_h + D, __float_as_uint(lse_l), through);
-      }
-    }
-    return;
-  }
   uint16_t* out = (uint16_t*)a.out;
   const uint16_t* r16 = (const uint16_t*)rows;
   const uint32_t* r32 = (const uint32_t*)rows;
-  const uint32_t lse16_l = f32_to_bits16(lse_l, a.mid_dtype);
+  // lane h serves row h's single values: its LSE (and, for a row that starts between two boundaries, value 0)
+  const int hl = lane < nheads ? lane : nheads - 1;
+  const float lse_l = empty ? -INFINITY : lse_slot[hl];
   const bool paired = !a.lse && !a.no_lse;
   if (!paired) {
     // 16-bit rows without an LSE behind them: element by element
@@ -916,80 +913,34 @@ __device__ __forceinline__ void wave_copy_parked(const SplitArgs& a, const char*
   }
   // element parity of a row's start relative to a 4-byte boundary
   const uint64_t par0 = (reinterpret_cast<uintptr_t>(a.out) >> 1) + (uint64_t)row0;
-  constexpr int NW = (D / 2 + 63) / 64;   // dwords per lane and row (D = 64: half the lanes are idle)
-  if ((a.so_h & 1) == 0) {
-    // The usual case -- an even number of splits, so that all heads of a split start with the same parity: one
-    // wave-uniform decision instead of one per row.
-    const bool first = (__builtin_amdgcn_readfirstlane((int)(par0 & 1))) != 0;
-    if (lane < nheads) {
-      uint16_t* row = out + row0 + (int64_t)hl * a.so_h;
-      store_bits16(row + (first ? 0 : D), first ? (empty ? 0u : (uint32_t)r16[hl * D]) : lse16_l, through);
-    }
-    for (int h0 = 0; h0 < nheads; h0 += 4) {
-      uint32_t lo[4][NW], hi[4][NW], lse16[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int hh = min(h0 + i, nheads - 1);
-        if (first) lse16[i] = f32_to_bits16(empty ? -INFINITY : lse_slot[hh], a.mid_dtype);
-#pragma unroll
-        for (int k = 0; k < NW; ++k) {
-          const int w = min(lane + 64 * k, D / 2 - 1);   // dword of the parked row: values 2 w, 2 w + 1
-          lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
-          if (first) hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (h0 + i >= nheads) break;
-        uint16_t* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
-#pragma unroll
-        for (int k = 0; k < NW; ++k) {
-          const int w = lane + 64 * k;
-          if (w >= D / 2) continue;
-          if (first) {   // values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
-            const uint32_t next = w == D / 2 - 1 ? lse16[i] : hi[i][k];
-            store_bits32(row + 2 * w + 1, (lo[i][k] >> 16) | (next << 16), through);
-          } else {
-            store_bits32(row + 2 * w, lo[i][k], through);
-          }
-        }
-      }
-    }
-    return;
-  }
   if (lane < nheads) {
     const bool first_l = ((par0 + (uint64_t)hl * (uint64_t)a.so_h) & 1) != 0;
     uint16_t* row = out + row0 + (int64_t)hl * a.so_h;
-    store_bits16(row + (first_l ? 0 : D), first_l ? (empty ? 0u : (uint32_t)r16[hl * D]) : lse16_l, through);
+    store_bits16(row + (first_l ? 0 : D), first_l ? (empty ? 0u : (uint32_t)r16[hl * D]) : f32_to_bits16(lse_l, a.mid_dtype),
+                 through);
   }
-  for (int h0 = 0; h0 < nheads; h0 += 4) {
-    uint32_t lo[4][NW], hi[4][NW], lse16[4];
-    int first[4];
+  const int j = lane % LPR;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int hh = min(h0 + i, nheads - 1);
-      first[i] = (int)((par0 + (uint64_t)hh * (uint64_t)a.so_h) & 1);
-      lse16[i] = (uint32_t)__shfl((int)lse16_l, hh);
-#pragma unroll
-      for (int k = 0; k < NW; ++k) {
-        const int w = min(lane + 64 * k, D / 2 - 1);   // dword of the parked row: values 2 w, 2 w + 1
-        lo[i][k] = empty ? 0u : r32[hh * (D / 2) + w];
-        hi[i][k] = empty ? 0u : r32[hh * (D / 2) + min(w + 1, D / 2 - 1)];
-      }
+  for (int r = 0; r < HB / RPS; ++r) {
+    const int h = r * RPS + lane / LPR;
+    if (h >= nheads) continue;
+    const uint32_t first = (uint32_t)((par0 + (uint64_t)h * (uint64_t)a.so_h) & 1);
+    u32x4 w = {0u, 0u, 0u, 0u};
+    uint32_t next = 0u;
+    if (!empty) {
+      w = *(const u32x4*)(r32 + h * (D / 2) + 4 * j);
+      next = r32[h * (D / 2) + min(4 * j + 4, D / 2 - 1)];
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (h0 + i >= nheads) break;
-      uint16_t* row = out + row0 + (int64_t)(h0 + i) * a.so_h;
-#pragma unroll
-      for (int k = 0; k < NW; ++k) {
-        const int w = lane + 64 * k;
-        if (w >= D / 2) continue;
-        // a row that starts between two boundaries: values (2 w + 1, 2 w + 2), the last pair (D - 1, LSE)
-        const uint32_t next = w == D / 2 - 1 ? lse16[i] : (hi[i][k] & 0xffffu);
-        const uint32_t word = first[i] ? (lo[i][k] >> 16) | (next << 16) : lo[i][k];
-        store_bits32(row + 2 * w + first[i], word, through);
-      }
+    if (j == LPR - 1) next = f32_to_bits16(empty ? -INFINITY : lse_slot[h], a.mid_dtype);
+    if (first) {
+      w = u32x4{__builtin_amdgcn_alignbit(w[1], w[0], 16), __builtin_amdgcn_alignbit(w[2], w[1], 16),
+                __builtin_amdgcn_alignbit(w[3], w[2], 16), __builtin_amdgcn_alignbit(next, w[3], 16)};
+    }
+    uint16_t* p = out + row0 + (int64_t)h * a.so_h + 8 * j + first;
+    if (through) {
+      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(w) : "memory");
+    } else {
+      *(u32x4_a4*)p = w;
     }
   }
 }
