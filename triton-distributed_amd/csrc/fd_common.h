@@ -52,8 +52,8 @@ struct SplitArgs {
                       // heads than a wave serves: the blocks read the same K/V rows in step, so the rows come
                       // from HBM once)
   int32_t grid_x;   // workgroups per (sequence, split)
-  int32_t vec_out;  // 1: every out row starts on a multiple of four elements (one 128-bit store per four fp32 values, one
-                    // 64-bit store per four 16-bit values)
+  int32_t vec_out;  // 1: four values of an out row go out in one store -- fp32 rows (any 4-byte boundary will do for a
+                    // 128-bit store), 16-bit rows that start on multiples of four elements (64-bit stores)
   int32_t no_lse;   // 1: the partial LSE is not stored (single split written straight to a [B,Hq,D] output)
   uint32_t s_magic, s_shift;      // n / S, same scheme as div_magic
   int32_t per_mask;               // split_align - 1 (0: the reference's ranges): tokens per split are rounded up
@@ -203,6 +203,11 @@ __device__ __forceinline__ float fd_softcap(float x, float cap, float inv_cap) {
 __device__ __forceinline__ u32x4 load_stream_b128(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
 __device__ __forceinline__ u32x2 load_stream_b64(const void* p) { return __builtin_nontemporal_load((const u32x2*)p); }
 
+// Vectors in global memory that are only known to start on a 4-byte boundary: global loads and stores of two or four
+// dwords need no more than dword alignment on this target.
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
 // Four consecutive values of a partial row that starts on a multiple of four elements (SplitArgs::vec_out): one
 // 128-bit store for fp32, one 64-bit store of four packed values for fp16 / bf16.  through: written through to memory
 // (sc0 sc1).  The write-through form is inline assembly, which the compiler does not count in vmcnt: only for stores
@@ -215,7 +220,7 @@ __device__ __forceinline__ void store_partial4(void* base, int64_t off, int dtyp
     if (through) {
       asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(o) : "memory");
     } else {
-      *(f32x4*)p = o;
+      *(f32x4_a4*)p = o;   // fp32 rows count as vector rows on any 4-byte boundary
     }
   } else {
     const f32x2 lo = {o[0], o[1]}, hi = {o[2], o[3]};
@@ -806,11 +811,6 @@ __device__ __forceinline__ uint32_t f32_to_bits16(float x, int dtype) {
   return dtype == FD_F16 ? (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x)
                          : (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
 }
-
-// Vectors in global memory that are only known to start on a 4-byte boundary: global loads and stores of two or four
-// dwords need no more than dword alignment on this target.
-typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 // Chunked work items: ONE wave copies a finished partial that it parked in LDS (HB fp32 LSEs, then the normalised
 // rows [head][D] of its real heads in mid_dtype) to split s of its head slots.  Called at the end of the wave's run
