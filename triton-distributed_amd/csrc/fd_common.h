@@ -325,6 +325,13 @@ __device__ __forceinline__ int tokens_per_range(int kv_len, int S, uint32_t s_ma
   return (per + per_mask) & ~per_mask;
 }
 
+// x / d for x >= 0 and a wave-uniform d > 0 that is a power of two in almost every launch (waves per range, members
+// per workgroup): a scalar test and a shift instead of the division sequence, which sits in front of the first table
+// lookup of every wave.
+__device__ __forceinline__ int div_uniform(int x, int d) {
+  return (d & (d - 1)) == 0 ? x >> (31 - __clz(d)) : x / d;
+}
+
 struct WorkItem {
   int b, s, kvh, hb, start, end;
   bool skip;  // empty range and nothing to write: the workgroup may leave at once (uniform over the workgroup)
@@ -363,6 +370,13 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
   }
   fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
+  // ... and the length is pinned like them: left alone, the compiler sinks its load below the index arithmetic that
+  // follows, to the block of its first use, and waits for it there -- one more dependent round trip in front of the
+  // first table lookup
+  {
+    const int len_now = (int)len;
+    asm volatile("" ::"s"(len_now));
+  }
 
   const int wave = threadIdx.x >> 6;
   if (a.member_hb) {
@@ -370,7 +384,7 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     const int groups = a.nhb / a.hpw;
     const int kvh = groups == 1 ? (int)blockIdx.x : (int)blockIdx.x / groups;
     const int hbg = blockIdx.x - kvh * groups;
-    w.sub = wave / a.hpw;
+    w.sub = div_uniform(wave, a.hpw);
     w.hb0 = hbg * a.hpw;
     w.hb = w.hb0 + (wave - w.sub * a.hpw);
     w.kvh0 = kvh;
@@ -391,14 +405,14 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
       w.kvh = grp;
       w.sub = wave;
     } else if (a.v_members == 2) {   // members are (KV head, V half) pairs: hpw / 2 heads per workgroup
-      const int member = wave - (wave / a.hpw) * a.hpw;
+      const int member = wave - div_uniform(wave, a.hpw) * a.hpw;
       w.kvh0 = grp * (a.hpw >> 1);
-      w.sub = wave / a.hpw;
+      w.sub = div_uniform(wave, a.hpw);
       w.kvh = w.kvh0 + (member >> 1);
       w.vh = member & 1;
     } else {
       w.kvh0 = grp * a.hpw;
-      w.sub = wave / a.hpw;
+      w.sub = div_uniform(wave, a.hpw);
       w.kvh = w.kvh0 + (wave - w.sub * a.hpw);
     }
     w.nsub = a.nsub;
@@ -410,7 +424,7 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
   w.per = per;
   if (a.chunk > 1) {
     // s counts work items of a.chunk splits; the waves of a head share them out in runs of whole splits
-    const int ns = (a.chunk + w.nsub - 1) / w.nsub;
+    const int ns = div_uniform(a.chunk + w.nsub - 1, w.nsub);
     const int first = s * a.chunk + w.sub * ns;
     const int lim = min(min((s + 1) * a.chunk, a.S), first + ns);
     w.s = first;

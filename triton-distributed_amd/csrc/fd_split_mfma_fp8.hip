@@ -56,7 +56,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) fd_split_mfma_fp8_kernel(
   if (CHUNK && w.ns <= 0) return;   // more waves than splits in the last work item of a sequence (no barrier follows)
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + kTile - 1) / kTile : 0;
-  const int tpw = (ntiles + w.nsub - 1) / w.nsub;
+  const int tpw = div_uniform(ntiles + w.nsub - 1, w.nsub);
   const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 

@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(512) fd_split_valu_kernel(const SplitArgs a) {
   if (w.skip) return;   // empty range, and the combine does not expect a partial from it
   const int ntok = w.end - w.start;
   const int ntiles = ntok > 0 ? (ntok + TILE - 1) / TILE : 0;
-  const int tpw = (ntiles + w.nsub - 1) / w.nsub;
+  const int tpw = div_uniform(ntiles + w.nsub - 1, w.nsub);
   const int t0 = w.sub * tpw;
   const int t1 = min(t0 + tpw, ntiles);
 
