@@ -30,6 +30,10 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     # packed-FP32 VALU ops are switched off for every device translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # Machine-code sinking off: the split kernels request a sequence's length right behind their argument batch and
+    # use it only after the index arithmetic of the work item; the sinking pass moves such a load down to the block of
+    # its first use, where the wave then waits a full round trip for it.
+    "-mllvm", "-disable-machine-sink",
     "-Wno-unused-command-line-argument",
 ]
 

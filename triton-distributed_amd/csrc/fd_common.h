@@ -369,15 +369,6 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     w.b = min(max(b, 0), a.batch - 1);
     len = a.order && a.order_lens ? a.order_lens[r] : a.kv_lens[w.b];
   }
-  fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
-  // ... and the length is pinned like them: left alone, the compiler sinks its load below the index arithmetic that
-  // follows, to the block of its first use, and waits for it there -- one more dependent round trip in front of the
-  // first table lookup
-  {
-    const int len_now = (int)len;
-    asm volatile("" ::"s"(len_now));
-  }
-
   const int wave = threadIdx.x >> 6;
   if (a.member_hb) {
     // workgroup = hpw head blocks of one KV head; blockIdx.x = kv head * (nhb / hpw) + block group
@@ -417,6 +408,15 @@ __device__ __forceinline__ WorkItem decode_work_item(const SplitArgs& a) {
     }
     w.nsub = a.nsub;
   }
+  fd_fetch_args_now(a);   // issued behind the loads above: the rest of the arguments arrives together with them
+  // ... and the length is pinned like them: left alone, the compiler sinks its load below the index arithmetic that
+  // follows, to the block of its first use, and waits for it there -- one more dependent round trip in front of the
+  // first table lookup
+  {
+    const int len_now = (int)len;
+    asm volatile("" ::"s"(len_now));
+  }
+
   int64_t cap = (int64_t)a.max_pages * a.P;
   len = len < 0 ? 0 : (len > cap ? cap : len);
   const int kv_len = (int)len;
