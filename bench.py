@@ -303,8 +303,8 @@ def measure_targets(torch, fd, dev, steps, warmup, c2_resident):
     c4 = U.make_config(4)
     n4 = steps // 4   # a step of config 4 is 15 times config 2's
     put("c4_ragged_scheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0, variant="persistent"))
-    # the plain wrapper ranks the sequences of a batch this large itself; "unscheduled" is that wrapper with the
-    # ranking switched off: sequences issued in index order
+    # the plain wrapper orders the work of a batch this large itself, as the scheduled one does; "unscheduled" is that
+    # wrapper with the ordering switched off: sequences issued in index order
     put("c4_ragged_plain_wrapper", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0))
     put("c4_ragged_unscheduled", measure_target(torch, fd, dev, c4, n4, 5, 2, 100.0, auto_order=False))
     del c4

@@ -263,7 +263,8 @@ typedef enum fd_step_flags {
                                  instead of the library's count; the partials still live in the workspace           */
   FD_STEP_SCHEDULE = 2,       /* the scheduled variant (gqa_fwd_batch_decode_persistent, flash_decode.py:931-1005):
                                  the step ranks its work on the device first -- (sequence, range) work items up to
-                                 192 sequences, whole sequences up to 4096 -- and issues it largest first             */
+                                 192 sequences, whole sequences up to 4096 -- and issues it largest first.  A step of
+                                 64 sequences or more does so whether this flag is set or not                        */
   FD_STEP_NO_ORDER = 4,       /* never rank: workgroups are issued in index order                                    */
   FD_STEP_FUSED = 8,          /* fd_plan_decode only: plan for fd_decode with a ticket buffer (fp32 partials, no
                                  work items, no direct single-split output)                                          */

@@ -347,11 +347,14 @@ def test_launch_plan_of_the_five_configs_and_the_published_sweep(fd):
         assert shape(lp) == (32, 0, 0, mid, 0, 0, 1, 32, 2, 2, 4, (4, 8, 8)) and lp.workspace_bytes == 0
     # config 3: one sequence of 131072 tokens + 7 extra partials
     assert shape(_plan(fd, 1, 32, 8, 32, 8192, extra=7)) == (64, 64, 64, F32, 0, 0, 1, 32, 2, 2, 1, (4, 1, 64))
-    # config 4: ragged batch of 64 -- the plain step ranks its sequences, the scheduled one its (sequence, range) items
-    lp = _plan(fd, 64, 32, 8, 32, 2048)
-    assert shape(lp) == (8, 1, 64, BF16, 0, L.FD_ORDER_SEQUENCES, 1, 32, 2, 2, 1, (4, 64, 8)) and lp.order_bytes == 256
-    lp = _plan(fd, 64, 32, 8, 32, 2048, flags=L.FD_STEP_SCHEDULE)
-    assert shape(lp) == (8, 1, 64, BF16, 0, L.FD_ORDER_ITEMS, 1, 32, 2, 2, 1, (4, 8, 64)) and lp.order_bytes == 2 * 64 * 8 * 4
+    # config 4: ragged batch of 64 -- from 64 sequences on a step orders its (sequence, range) items whether it was asked
+    # to or not; below that only when asked
+    for flags in (0, L.FD_STEP_SCHEDULE):
+        lp = _plan(fd, 64, 32, 8, 32, 2048, flags=flags)
+        assert shape(lp) == (8, 1, 64, BF16, 0, L.FD_ORDER_ITEMS, 1, 32, 2, 2, 1, (4, 8, 64)) and lp.order_bytes == 2 * 64 * 8 * 4
+    assert _plan(fd, 63, 32, 8, 32, 2048).order_kind == L.FD_ORDER_NONE
+    assert _plan(fd, 63, 32, 8, 32, 2048, flags=L.FD_STEP_SCHEDULE).order_kind == L.FD_ORDER_ITEMS
+    assert _plan(fd, 193, 32, 8, 32, 2048).order_kind == L.FD_ORDER_SEQUENCES   # beyond 192 sequences the per-sequence order
     assert _plan(fd, 64, 32, 8, 32, 2048, flags=L.FD_STEP_NO_ORDER).order_kind == L.FD_ORDER_NONE
     # config 5: fp8 cache, four sibling KV heads per workgroup; exactly 64 splits: written-through 16-bit partials
     assert shape(_plan(fd, 32, 64, 8, 64, 1024, kv=FP8)) == (4, 4, 64, BF16, 0, 0, 1, 64, 2, 4, 1, (2, 32, 4))

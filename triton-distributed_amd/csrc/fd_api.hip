@@ -1068,8 +1068,10 @@ int plan_step(const char* fn, const fd_params* in, int32_t batch, int32_t num_ex
   if (!caller_order && !(flags & FD_STEP_NO_ORDER) && batch > 1) {
     const bool free_order = (flags & FD_STEP_ORDER_FROM_APPEND) && batch >= kAppendOrderFromBatch;
     const bool scheduled = (flags & FD_STEP_SCHEDULE) || free_order;
-    const bool items = scheduled && S > 1 && !fused && batch <= kItemsUpToBatch;
     const bool ranked = scheduled || (batch >= kAutoOrderFromBatch && capacity >= kAutoOrderMinCapacity);
+    // (a step that ranks of its own accord takes the item list as well where it applies: over ragged batches of 72 ...
+    // 160 sequences it ran 1 - 4 % ahead of the per-sequence order, on config 4 650 against 687 us)
+    const bool items = ranked && S > 1 && !fused && batch <= kItemsUpToBatch;
     if (items) {
       r.order_kind = FD_ORDER_ITEMS;
       r.p.seq_order_items = 1;

@@ -15,8 +15,9 @@ Keyword-only additions that the reference does not have (all default off):
   extra_partials  (out [E,B,Hq,Dv], lse [E,B,Hq] fp32): further partials merged by
                   the combine, standing in for what other sequence-parallel ranks
                   would contribute
-  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (batches of 64 sequences or
-                  more are ranked by the step itself when none is given; ``auto_order=False`` switches that off)
+  seq_order       int32 [B] from ``schedule_sequences``: issue order of the sequences (a batch of 64 sequences or
+                  more orders its work itself when none is given -- (sequence, range) items up to 192 sequences,
+                  whole sequences beyond; ``auto_order=False`` switches that off)
   seq_order_lens  int32 [B], with ``seq_order``: ``kv_lens[seq_order]`` (``rope_kv_append`` writes both), which
                   saves a workgroup one dependent load before it can start
   path            "auto" | "valu" | "mfma"; waves_per_block 0 | 1 | 2 | 4 | 8
