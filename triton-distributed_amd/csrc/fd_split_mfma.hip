@@ -111,7 +111,13 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
     return bt_row[pidx];
   };
 
-  u32x4 kraw[8], vraw[8];
+  // VEARLY (two head blocks per wave, one workgroup per split): a tile's compute is long enough there that a V tile
+  // requested only when its predecessor has been consumed leaves the wave with half its bytes in flight for most of
+  // the tile.  V gets a second register set instead, and V(t+1) is requested together with K(t+1) at the start of
+  // tile t; the tiles of a run alternate between the sets (compile-time parity, the loop is unrolled by two).
+  constexpr bool VEARLY = NB == 2 && !CHUNK;
+  constexpr int VB = VEARLY ? 2 : 1;
+  u32x4 kraw[8], vraw[VB][8];
   int rows[8];
   auto fetch_rows = [&](int page, int slot) {
     // flat cache row = page * P + slot, page clamped into the pool so a corrupt table cannot fault
@@ -123,9 +129,10 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
 #pragma unroll
     for (int i = 0; i < 8; ++i) kraw[i] = load_stream_b128(kbase + (int64_t)rows[i] * k_pitch);
   };
-  auto issue_v = [&]() {
+  auto issue_v = [&](auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) vraw[i] = load_stream_b128(vbase + (int64_t)rows[i] * v_pitch);
+    for (int i = 0; i < 8; ++i) vraw[SET][i] = load_stream_b128(vbase + (int64_t)rows[i] * v_pitch);
   };
 
   float m[NB];          // running max of head 16*nb + c (identical in the 4 wave rows)
@@ -146,8 +153,11 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
   // K(t+1) and V(t+1) are in flight while tile t is being computed.
   // n0 / n_end: first token of the tile and end of its split (for the mask); lookup2(slot): table entry and slot of
   // this lane's token two tiles ahead.
-  auto tile = [&](const int n0, const int n_end, auto&& lookup2, auto has_next_tag) {
+  // set_tag: the V register set that holds this tile (always 0 without VEARLY).
+  auto tile = [&](const int n0, const int n_end, auto&& lookup2, auto has_next_tag, auto set_tag) {
     constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+    constexpr int SET = decltype(set_tag)::value;
+    static_assert(SET < VB, "V register set");
     // ---- K tile -> LDS, then start fetching the next tile's K into the freed registers
     wave_lds_fence();
 #pragma unroll
@@ -162,6 +172,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       __builtin_amdgcn_sched_barrier(0);
       fetch_rows(pg_next, slot_next);
       issue_k();
+      if constexpr (VEARLY) issue_v(std::integral_constant<int, (SET ^ 1) & (VB - 1)>{});
       pg_next = lookup2(slot_next);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -228,12 +239,12 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
         const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          vop[jj][e] = __builtin_amdgcn_perm(vraw[2 * e + 1][j >> 1], vraw[2 * e][j >> 1], sel);
+          vop[jj][e] = __builtin_amdgcn_perm(vraw[SET][2 * e + 1][j >> 1], vraw[SET][2 * e][j >> 1], sel);
       }
-      if constexpr (HAS_NEXT) {
+      if constexpr (HAS_NEXT && !VEARLY) {
         if (j0 + kHalf == 8) {
           __builtin_amdgcn_sched_barrier(0);
-          issue_v();
+          issue_v(set_tag);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -328,11 +339,11 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       __builtin_amdgcn_sched_barrier(0);
       fetch_rows(pg0, slot0);
       issue_k();
-      issue_v();
+      issue_v(std::integral_constant<int, 0>{});
       __builtin_amdgcn_sched_barrier(0);
       auto lookup2 = [&](int& slot) -> int { return token_slot(look.base, look.end, slot); };
       while (!(cur.end >= run_end && cur.base + kTile >= cur.end)) {   // all tiles but the wave's last one
-        tile(cur.base, cur.end, lookup2, std::true_type{});
+        tile(cur.base, cur.end, lookup2, std::true_type{}, std::integral_constant<int, 0>{});
         if (cur.base + kTile >= cur.end) {   // that was the last tile of a split
           park_final(park + parked * a.park_bytes);
           ++parked;
@@ -347,7 +358,7 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
         cur = advance(cur);
         look = advance(look);
       }
-      tile(cur.base, cur.end, lookup2, std::false_type{});
+      tile(cur.base, cur.end, lookup2, std::false_type{}, std::integral_constant<int, 0>{});
       park_final(kb);   // the wave's last split: its staging buffer is free now
       last_staged = true;
     }
@@ -366,13 +377,34 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
       __builtin_amdgcn_sched_barrier(0);
       fetch_rows(pg0, slot0);
       issue_k();
-      issue_v();
+      issue_v(std::integral_constant<int, 0>{});
       __builtin_amdgcn_sched_barrier(0);
-      for (int t = t0; t < t1 - 1; ++t)
+      using Set0 = std::integral_constant<int, 0>;
+      using Set1 = std::integral_constant<int, VB - 1>;   // the other V register set, if there is one
+      auto inner = [&](int t, auto set_tag) {   // a tile that has a successor
         tile(w.start + t * kTile, w.end, [&](int& slot) -> int { return tile_slot(min(t + 2, t1 - 1), slot); },
-             std::true_type{});
-      tile(w.start + (t1 - 1) * kTile, w.end, [&](int& slot) -> int { return tile_slot(t1 - 1, slot); },
-           std::false_type{});
+             std::true_type{}, set_tag);
+      };
+      auto last = [&](auto set_tag) {
+        tile(w.start + (t1 - 1) * kTile, w.end, [&](int& slot) -> int { return tile_slot(t1 - 1, slot); },
+             std::false_type{}, set_tag);
+      };
+      if constexpr (VEARLY) {
+        int t = t0;
+        for (; t + 2 < t1; t += 2) {
+          inner(t, Set0{});
+          inner(t + 1, Set1{});
+        }
+        if (t + 1 < t1) {   // two tiles left
+          inner(t, Set0{});
+          last(Set1{});
+        } else {
+          last(Set0{});
+        }
+      } else {
+        for (int t = t0; t < t1 - 1; ++t) inner(t, Set0{});
+        last(Set0{});
+      }
     }
 
     // ---- wave result -> LDS, then workgroup merge
