@@ -114,7 +114,9 @@ __global__ void __launch_bounds__(NB == 2 ? 256 : 512) FD_MFMA_OCC fd_split_mfma
   // VEARLY (two head blocks per wave, one workgroup per split): a tile's compute is long enough there that a V tile
   // requested only when its predecessor has been consumed leaves the wave with half its bytes in flight for most of
   // the tile.  V gets a second register set instead, and V(t+1) is requested together with K(t+1) at the start of
-  // tile t; the tiles of a run alternate between the sets (compile-time parity, the loop is unrolled by two).
+  // tile t; the tiles of a run alternate between the sets (compile-time parity, the loop is unrolled by two).  With one
+  // head block per wave the same change loses: that kernel streams at what the memory gives, and more requests in
+  // flight only lengthen the queues (config 2 44.4 -> 45.1 us, a 131072-token sequence 84.8 -> 86.1 us).
   constexpr bool VEARLY = NB == 2 && !CHUNK;
   constexpr int VB = VEARLY ? 2 : 1;
   u32x4 kraw[8], vraw[VB][8];
