@@ -830,9 +830,8 @@ __device__ __forceinline__ uint32_t f32_to_bits16(float x, int dtype) {
 // rows [head][D] of its real heads in mid_dtype) to split s of its head slots.  Called at the end of the wave's run
 // only: on this target stores and loads of a wave retire in order (one vmcnt), so a store issued between two tiles
 // would hold back every later K/V load until it is acknowledged.  empty: the split holds no token (out = 0,
-// lse = -inf; the slot is not read).  Every form moves 128 bits per lane (64 for 16-bit rows on multiples of four
-// elements) with whole rows per store instruction, and the values are the parked bits: nothing is scaled or
-// converted here but the LSE.
+// lse = -inf; the slot is not read).  Every form moves 128 bits per lane with whole rows per store instruction, and
+// the values are the parked bits: nothing is scaled or converted here but the LSE.
 //  * fp32 rows, and 16-bit rows that start on multiples of four elements (the library's own layout): straight copies.
 //    fp32 rows of the reference's [B, Hq, S, D + 1] layout start on 4-byte boundaries only, which is all a 128-bit
 //    store needs.
